@@ -1,0 +1,86 @@
+// Shared definitions for the gfx950 FlashAttention-forward kernels: launch-argument structs, vector types,
+// wave64 helpers and the counter-based Philox used for dropout.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fa {
+
+typedef _Float16 half_t;
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+// operand type of the ds_read_b64_tr_b16 builtin
+typedef __fp16 v4hp __attribute__((__vector_size__(4 * sizeof(__fp16))));
+
+#define FA_LDS __attribute__((address_space(3)))
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Arguments of the tiled forward kernel and of the decode/combine kernels, filled by the host from flash_params
+// (which is itself the superset of the reference's mykernelParamType, include/utils.h:21-44).
+struct FwdArgs {
+    const half_t* Q;
+    const half_t* K;
+    const half_t* V;
+    half_t* O;
+    float* LSE;
+    float* O_partial;    // [B,H,S,Nq,d] fp32, normalised per split (reference O_tmp)
+    float* LSE_partial;  // [B,H,S,Nq]   fp32, m_s + log l_s   (reference M, L)
+    const float* alibi;  // [H] or nullptr
+    uint8_t* keep_out;   // [B,H,Nq,Nk] or nullptr
+    int B, H, Nq, Nk, d;
+    int causal, wl, wr;  // wl / wr < 0: unbounded
+    float scale_log2;    // softmax_scale * log2(e)
+    uint32_t drop_thr;   // keep iff philox word >= drop_thr
+    float drop_rscale;   // 1 / (1 - p)
+    uint32_t seed_lo, seed_hi, off_lo;
+    int num_splits;      // 1: write O/LSE; > 1: write the partial workspace
+    int keys_per_split;  // multiple of 128
+    int Tr;              // number of query row blocks
+};
+
+__device__ __forceinline__ int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// Exchange between lane l and lane l^32 (v_permlane32_swap): result[0] holds the low half's value in both halves,
+// result[1] the high half's.
+__device__ __forceinline__ float xhalf_max(float v)
+{
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xhalf_sum(float v)
+{
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// Philox4x32-10.  Dropout contract: key = (lo32(seed), hi32(seed)); counter = (j >> 2, i, b*H + h, lo32(offset));
+// element (i, j) uses output word j & 3 and is kept iff word >= floor(p * 2^32).  Replaces the stateful
+// curandStatePhilox4_32_10_t draw of the reference (src/flash_forward.h:50-54,227).
+__device__ __forceinline__ v4u philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1)
+{
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+        const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+        c0 = hi1 ^ c1 ^ k0;
+        c1 = lo1;
+        c2 = hi0 ^ c3 ^ k1;
+        c3 = lo0;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    v4u o = {c0, c1, c2, c3};
+    return o;
+}
+
+}  // namespace fa

@@ -1,0 +1,259 @@
+// Split-KV decode (one query row per head), split combine, and the stand-alone dropout keep-mask kernel.
+//
+// decode_split_kernel replaces forward_kernel_splitkv (src/flash_forward_splitkv.h:14-344) for Nq == 1, where the
+// reference's 128-row MMA tile would waste 127 of 128 rows: the work is a pure stream over K and V, bound by HBM.
+//   * one work-group per (head slice, split); its 4 waves take 128-byte-per-lane blocks of the split's keys in turn
+//   * a key row is spread over LPK lanes (16 bytes each), so one wave instruction reads 1 KiB of consecutive bytes
+//   * q.k: v_dot2_f32_f16 per lane, then a DPP butterfly over the LPK lanes of the key (no LDS, no shuffles)
+//   * online softmax per key group; p * V accumulated in fp32 per lane (8 head-dim columns per lane)
+//   * key groups and waves are merged once at the end through LDS; partial O (normalised, fp32) and
+//     LSE_s = m_s + log l_s go to the workspace (reference: O_tmp, M, L; src/flash_forward_splitkv.h:313-338)
+// combine_kernel replaces forward_kernel_splitkv_combine (src/flash_forward_splitkv.h:347-399) with one wave per
+// query row and coalesced reads of the partials (the reference uses one thread per row).
+#include "common.h"
+#include "decode_kernels.h"
+
+namespace fa {
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+// sum over the LPK consecutive lanes that share a key; every lane of the group ends with the total
+template <int LPK>
+__device__ __forceinline__ float group_sum(float v)
+{
+    v += dpp_mov<0xB1>(v);                          // quad_perm [1,0,3,2]
+    v += dpp_mov<0x4E>(v);                          // quad_perm [2,3,0,1]
+    if constexpr (LPK >= 8) v += dpp_mov<0x141>(v);   // row_half_mirror
+    if constexpr (LPK >= 16) v += dpp_mov<0x140>(v);  // row_mirror
+    return v;
+}
+
+template <int LPK, bool kAlibi>
+__global__ void __launch_bounds__(256) decode_split_kernel(const FwdArgs a)
+{
+    constexpr int KPI = 64 / LPK;  // keys per wave instruction
+    constexpr int U = 8;           // load instructions in flight per tensor
+    constexpr int KB = U * KPI;    // keys per wave block
+    constexpr int NG = 4 * KPI;    // key groups per work-group
+    constexpr int DB = LPK * 8;    // head-dim bucket
+    __shared__ float s_acc[NG][DB];
+    __shared__ float s_m[NG], s_l[NG];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int c = lane % LPK;
+    const int kg = lane / LPK;
+    const int BH = a.B * a.H;
+    const int bh = blockIdx.x % BH;
+    const int split = blockIdx.x / BH;
+    const int h = bh % a.H;
+    const int d = a.d, Nk = a.Nk;
+    const int col = 8 * c;
+    const bool cvalid = col < d;
+    const int colc = cvalid ? col : d - 8;
+
+    union U8 { v4u u; v8h h; v2h p[4]; };
+    U8 qv;
+    qv.u = *reinterpret_cast<const v4u*>(a.Q + (size_t)bh * d + colc);
+    if (!cvalid) qv.u = v4u{0u, 0u, 0u, 0u};
+
+    // the single query row sits at position ii = Nk - 1 (row index i + Nk - Nq): causal / right window never cut
+    const int ii = Nk - 1;
+    int kstart = a.wl >= 0 ? max(0, ii - a.wl) : 0;
+    int kend = Nk;
+    if (a.num_splits > 1) {
+        kstart = max(kstart, split * a.keys_per_split);
+        kend = min(kend, (split + 1) * a.keys_per_split);
+    }
+    const half_t* __restrict__ Kbh = a.K + (size_t)bh * Nk * d + colc;
+    const half_t* __restrict__ Vbh = a.V + (size_t)bh * Nk * d + colc;
+    const float c2 = a.scale_log2;
+    float slope2 = 0.0f;
+    if constexpr (kAlibi) slope2 = a.alibi ? a.alibi[h] * kLog2e : 0.0f;
+
+    float m = -INFINITY, l = 0.0f;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+
+    for (int kb = kstart + wave * KB; kb < kend; kb += 4 * KB) {
+        U8 kr[U], vr[U];
+#pragma unroll
+        for (int i = 0; i < U; ++i) {
+            const int j = kb + i * KPI + kg;
+            const size_t off = (size_t)(j < kend ? j : kend - 1) * d;
+            kr[i].u = *reinterpret_cast<const v4u*>(Kbh + off);
+        }
+#pragma unroll
+        for (int i = 0; i < U; ++i) {
+            const int j = kb + i * KPI + kg;
+            const size_t off = (size_t)(j < kend ? j : kend - 1) * d;
+            vr[i].u = *reinterpret_cast<const v4u*>(Vbh + off);
+        }
+        float t[U];
+        float mb = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < U; ++i) {
+            float s = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s = __builtin_amdgcn_fdot2(qv.p[e], kr[i].p[e], s, false);
+            s = group_sum<LPK>(s);
+            const int j = kb + i * KPI + kg;
+            float tv = s * c2;
+            if constexpr (kAlibi) tv -= slope2 * (float)(ii - j);
+            if (j >= kend) tv = -INFINITY;
+            t[i] = tv;
+            mb = fmaxf(mb, tv);
+        }
+        const float m_new = fmaxf(m, mb);
+        const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+        const float alpha = fast_exp2(m - m_use);
+        m = m_new;
+        float rs = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] *= alpha;
+#pragma unroll
+        for (int i = 0; i < U; ++i) {
+            const float p = fast_exp2(t[i] - m_use);
+            rs += p;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(p, (float)vr[i].h[e], acc[e]);
+        }
+        l = l * alpha + rs;
+    }
+
+    // ---- merge the NG key groups of the work-group
+    const int grp = wave * KPI + kg;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s_acc[grp][col + e] = acc[e];
+    if (c == 0) {
+        s_m[grp] = m;
+        s_l[grp] = l;
+    }
+    __syncthreads();
+    if (tid < DB) {
+        float M = -INFINITY;
+#pragma unroll
+        for (int gI = 0; gI < NG; ++gI) M = fmaxf(M, s_m[gI]);
+        const float Mu = (M == -INFINITY) ? 0.0f : M;
+        float L = 0.0f, o = 0.0f;
+#pragma unroll
+        for (int gI = 0; gI < NG; ++gI) {
+            const float w = fast_exp2(s_m[gI] - Mu);
+            L += w * s_l[gI];
+            o += w * s_acc[gI][tid];
+        }
+        const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+        const float lse = L > 0.0f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
+        if (a.num_splits > 1) {
+            const size_t prow = (size_t)bh * a.num_splits + split;  // Nq == 1
+            if (tid < d) a.O_partial[prow * d + tid] = o * inv;
+            if (tid == 0) a.LSE_partial[prow] = lse;
+        } else {
+            if (tid < d) a.O[(size_t)bh * d + tid] = (half_t)(o * inv);
+            if (tid == 0) a.LSE[bh] = lse;
+        }
+    }
+}
+
+// One wave per query row: LSE = logsumexp_s LSE_s, O = sum_s exp(LSE_s - LSE) O_s
+// (same value as m = max M_s, l = sum e^{M_s-m} L_s, O = sum (L_s e^{M_s-m} / l) O_s of splitkv.h:359-397).
+__global__ void __launch_bounds__(256) combine_kernel(const float* __restrict__ O_partial,
+                                                      const float* __restrict__ LSE_partial, half_t* __restrict__ O,
+                                                      float* __restrict__ LSE, int BH, int Nq, int d, int S)
+{
+    __shared__ float s_w[4][FLASH_MAX_SPLITS_K];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const long long row = (long long)blockIdx.x * 4 + wave;
+    const long long rows = (long long)BH * Nq;
+    const bool valid = row < rows;
+    const int bh = valid ? (int)(row / Nq) : 0, i = valid ? (int)(row % Nq) : 0;
+    const float* lp = LSE_partial + (size_t)bh * S * Nq + i;  // stride Nq between splits
+    float mx = -INFINITY;
+    for (int s = lane; s < S; s += 64) mx = fmaxf(mx, lp[(size_t)s * Nq]);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    const float mu = (mx == -INFINITY) ? 0.0f : mx;
+    float sum = 0.0f;
+    for (int s = lane; s < S; s += 64) {
+        const float w = __expf(lp[(size_t)s * Nq] - mu);
+        s_w[wave][s] = w;
+        sum += w;
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o, 64);
+    const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
+    __syncthreads();
+    if (!valid) return;
+    for (int dc = lane; dc < d; dc += 64) {
+        float o = 0.0f;
+        for (int s = 0; s < S; ++s) o += s_w[wave][s] * O_partial[(((size_t)bh * S + s) * Nq + i) * d + dc];
+        O[((size_t)bh * Nq + i) * d + dc] = (half_t)(o * inv);
+    }
+    if (lane == 0) LSE[(size_t)bh * Nq + i] = sum > 0.0f ? mx + __logf(sum) : -INFINITY;
+}
+
+// keep[b,h,i,j] = philox word (j & 3) of counter (j >> 2, i, b*H + h, lo32(offset)) >= threshold
+__global__ void __launch_bounds__(256) keep_mask_kernel(uint8_t* __restrict__ mask, long long rows, int Nq, int Nk,
+                                                        uint32_t thr, uint32_t seed_lo, uint32_t seed_hi,
+                                                        uint32_t off_lo)
+{
+    const int groups = (Nk + 3) >> 2;
+    const long long total = rows * groups;
+    for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (long long)gridDim.x * 256) {
+        const long long r = idx / groups;
+        const int jg = (int)(idx % groups);
+        const uint32_t bh = (uint32_t)(r / Nq), i = (uint32_t)(r % Nq);
+        const v4u w = philox4x32_10((uint32_t)jg, i, bh, off_lo, seed_lo, seed_hi);
+        uint8_t* mrow = mask + (size_t)r * Nk;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (4 * jg + e < Nk) mrow[4 * jg + e] = w[e] >= thr ? 1 : 0;
+    }
+}
+
+int launch_decode_split(const FwdArgs& a, hipStream_t st)
+{
+    const unsigned groups = (unsigned)((long long)a.B * a.H * a.num_splits);
+    const bool alibi = a.alibi != nullptr;
+    if (a.d > 64) {
+        if (alibi) hipLaunchKernelGGL((decode_split_kernel<16, true>), dim3(groups), dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((decode_split_kernel<16, false>), dim3(groups), dim3(256), 0, st, a);
+    } else if (a.d > 32) {
+        if (alibi) hipLaunchKernelGGL((decode_split_kernel<8, true>), dim3(groups), dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((decode_split_kernel<8, false>), dim3(groups), dim3(256), 0, st, a);
+    } else {
+        if (alibi) hipLaunchKernelGGL((decode_split_kernel<4, true>), dim3(groups), dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((decode_split_kernel<4, false>), dim3(groups), dim3(256), 0, st, a);
+    }
+    return (int)hipGetLastError();
+}
+
+int launch_combine(const FwdArgs& a, hipStream_t st)
+{
+    const long long rows = (long long)a.B * a.H * a.Nq;
+    const unsigned groups = (unsigned)((rows + 3) / 4);
+    hipLaunchKernelGGL(combine_kernel, dim3(groups), dim3(256), 0, st, a.O_partial, a.LSE_partial, a.O, a.LSE,
+                       a.B * a.H, a.Nq, a.d, a.num_splits);
+    return (int)hipGetLastError();
+}
+
+int launch_keep_mask(uint8_t* mask, int B, int H, int Nq, int Nk, uint32_t thr, uint64_t seed, uint64_t offset,
+                     hipStream_t st)
+{
+    const long long rows = (long long)B * H * Nq;
+    const long long total = rows * ((Nk + 3) / 4);
+    long long groups = (total + 255) / 256;
+    if (groups > 65536) groups = 65536;
+    if (groups < 1) groups = 1;
+    hipLaunchKernelGGL(keep_mask_kernel, dim3((unsigned)groups), dim3(256), 0, st, mask, rows, Nq, Nk, thr,
+                       (uint32_t)seed, (uint32_t)(seed >> 32), (uint32_t)offset);
+    return (int)hipGetLastError();
+}
+
+}  // namespace fa

@@ -1,0 +1,241 @@
+// C ABI of the library (include/flash_attn_mi355.h): argument checking, split resolution and kernel dispatch.
+// Host counterpart of the launch logic in the reference's main() (src/main.cu:109-192): fill the launch
+// arguments, pick the kernel, size the grid, enqueue (+ combine when the key range is split).
+#include "flash_attn_mi355.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+
+#include "common.h"
+#include "decode_kernels.h"
+#include "fwd_kernel.h"
+
+static_assert(FLASH_MAX_SPLITS == FLASH_MAX_SPLITS_K, "split limits out of sync");
+
+namespace {
+
+thread_local char g_hip_error[256] = "";
+
+int record_hip(int e)
+{
+    if (e == (int)hipSuccess) return FLASH_OK;
+    std::snprintf(g_hip_error, sizeof(g_hip_error), "%s", hipGetErrorString((hipError_t)e));
+    return FLASH_ELAUNCH;
+}
+
+constexpr int kNumCU = 256;  // MI355X
+
+inline bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
+
+// shape / scalar checks shared by every entry point; *empty is set when there is nothing to compute
+int validate_shape(const flash_params* p, bool* empty)
+{
+    *empty = false;
+    if (!p) return FLASH_EINVAL;
+    if (p->B < 0 || p->H < 0 || p->Nq < 0 || p->Nk < 0 || p->d <= 0) return FLASH_EINVAL;
+    if (p->d > FLASH_MAX_HEAD_DIM) return FLASH_EHEADDIM;
+    if (!(p->softmax_scale == p->softmax_scale) || std::isinf(p->softmax_scale)) return FLASH_EINVAL;
+    if (!(p->dropout_p >= 0.0f && p->dropout_p < 1.0f)) return FLASH_EINVAL;
+    if (p->num_splits > FLASH_MAX_SPLITS) return FLASH_ESPLITS;
+    if ((long long)p->B * p->H > 0x7fffffffLL / 2) return FLASH_EINVAL;
+    if (p->B == 0 || p->H == 0 || p->Nq == 0) *empty = true;
+    return FLASH_OK;
+}
+
+// pointer checks of the two launching entry points
+int validate(const flash_params* p, bool* empty)
+{
+    const int rc = validate_shape(p, empty);
+    if (rc != FLASH_OK || *empty) return rc;
+    if (!p->Q || !p->O || !p->LSE) return FLASH_EINVAL;
+    if (p->Nk > 0 && (!p->K || !p->V)) return FLASH_EINVAL;
+    // The vector path moves 16 bytes at a time, as the reference's cp.async does (include/utils.h:63).
+    const size_t need = (p->d % 8 == 0) ? 16 : 2;
+    if (misaligned(p->Q, need) || misaligned(p->O, need) || misaligned(p->LSE, 4)) return FLASH_EALIGN;
+    if (p->Nk > 0 && (misaligned(p->K, need) || misaligned(p->V, need))) return FLASH_EALIGN;
+    if (p->alibi_slopes && misaligned(p->alibi_slopes, 4)) return FLASH_EALIGN;
+    return FLASH_OK;
+}
+
+constexpr int kRowsPerGroup = 128;  // FwdCfg<D, 1>::BR
+
+void fill_args(const flash_params* p, int splits, fa::FwdArgs* a)
+{
+    std::memset(a, 0, sizeof(*a));
+    a->Q = static_cast<const fa::half_t*>(p->Q);
+    a->K = static_cast<const fa::half_t*>(p->K);
+    a->V = static_cast<const fa::half_t*>(p->V);
+    a->O = static_cast<fa::half_t*>(p->O);
+    a->LSE = p->LSE;
+    a->O_partial = p->O_partial;
+    a->LSE_partial = p->LSE_partial;
+    a->alibi = p->alibi_slopes;
+    a->keep_out = p->dropout_p > 0.0f ? p->keep_mask_out : nullptr;
+    a->B = p->B;
+    a->H = p->H;
+    a->Nq = p->Nq;
+    a->Nk = p->Nk;
+    a->d = p->d;
+    a->causal = p->is_causal ? 1 : 0;
+    a->wl = p->window_left;
+    a->wr = p->window_right;
+    a->scale_log2 = p->softmax_scale * fa::kLog2e;
+    a->drop_thr = flash_dropout_threshold(p->dropout_p);
+    a->drop_rscale = 1.0f / (1.0f - p->dropout_p);
+    a->seed_lo = (uint32_t)p->seed;
+    a->seed_hi = (uint32_t)(p->seed >> 32);
+    a->off_lo = (uint32_t)p->offset;
+    a->num_splits = splits;
+    const int blocks = (p->Nk + FLASH_SPLIT_KEY_GRANULE - 1) / FLASH_SPLIT_KEY_GRANULE;
+    a->keys_per_split = ((blocks + splits - 1) / splits) * FLASH_SPLIT_KEY_GRANULE;  // splitkv.h:40-43
+    a->Tr = (p->Nq + kRowsPerGroup - 1) / kRowsPerGroup;
+}
+
+int launch_tiled(const flash_params* p, const fa::FwdArgs& a, hipStream_t st)
+{
+    int variant = (p->d % 8 == 0) ? 1 : 0;
+    // a non-positive scale does not commute with the row maximum: take the variant that scales first
+    if (p->alibi_slopes || !(p->softmax_scale > 0.0f)) variant |= 2;
+    if (p->dropout_p > 0.0f) variant |= 4;
+    int e;
+    if (p->d <= 32) e = fa::launch_fwd_d32(a, variant, 1, st);
+    else if (p->d <= 64) e = fa::launch_fwd_d64(a, variant, 1, st);
+    else if (p->d <= 96) e = fa::launch_fwd_d96(a, variant, 1, st);
+    else e = fa::launch_fwd_d128(a, variant, 1, st);
+    return record_hip(e);
+}
+
+int resolve_splits(const flash_params* p)
+{
+    const int n_blocks = (p->Nk + FLASH_SPLIT_KEY_GRANULE - 1) / FLASH_SPLIT_KEY_GRANULE;
+    int s = p->num_splits;
+    if (s <= 0) {
+        const int Tr = (p->Nq + kRowsPerGroup - 1) / kRowsPerGroup;
+        // argument roles as in the reference's call (src/main.cu:125), with the CU count of the MI355X
+        s = flash_num_splits_heuristic(Tr * p->H * p->B, kNumCU, n_blocks, FLASH_MAX_SPLITS, n_blocks * FLASH_SPLIT_KEY_GRANULE);
+    }
+    if (s > n_blocks) s = n_blocks;  // never more splits than key blocks
+    if (s > FLASH_MAX_SPLITS) s = FLASH_MAX_SPLITS;
+    if (s < 1) s = 1;
+    return s;
+}
+
+}  // namespace
+
+#define FLASH_EXPORT __attribute__((visibility("default")))
+
+extern "C" {
+
+FLASH_EXPORT int flash_forward(const flash_params* p, void* stream)
+{
+    bool empty;
+    const int rc = validate(p, &empty);
+    if (rc != FLASH_OK || empty) return rc;
+    fa::FwdArgs a;
+    fill_args(p, 1, &a);
+    return launch_tiled(p, a, static_cast<hipStream_t>(stream));
+}
+
+FLASH_EXPORT int flash_forward_splitkv(const flash_params* p, void* stream)
+{
+    bool empty;
+    const int rc = validate(p, &empty);
+    if (rc != FLASH_OK || empty) return rc;
+    const int splits = resolve_splits(p);
+    if (splits > 1 && (!p->O_partial || !p->LSE_partial)) return FLASH_EWORKSPACE;
+    if (splits > 1 && (misaligned(p->O_partial, 16) || misaligned(p->LSE_partial, 4))) return FLASH_EALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    fa::FwdArgs a;
+    fill_args(p, splits, &a);
+    int e;
+    // one query row per head, 16-byte rows, no dropout: bandwidth-bound streaming kernel; otherwise the tiled kernel
+    if (p->Nq == 1 && p->d % 8 == 0 && p->dropout_p == 0.0f && p->softmax_scale > 0.0f)
+        e = record_hip(fa::launch_decode_split(a, st));
+    else
+        e = launch_tiled(p, a, st);
+    if (e != FLASH_OK || splits == 1) return e;
+    return record_hip(fa::launch_combine(a, st));
+}
+
+FLASH_EXPORT int flash_splitkv_resolve_splits(const flash_params* p)
+{
+    bool empty;
+    const int rc = validate_shape(p, &empty);
+    if (rc != FLASH_OK) return rc;
+    return empty ? 1 : resolve_splits(p);
+}
+
+FLASH_EXPORT int flash_splitkv_workspace_bytes(const flash_params* p, size_t* o_partial_bytes, size_t* lse_partial_bytes)
+{
+    bool empty;
+    const int rc = validate_shape(p, &empty);
+    if (rc != FLASH_OK) return rc;
+    const int splits = empty ? 1 : resolve_splits(p);
+    const size_t rows = splits > 1 ? (size_t)p->B * p->H * splits * p->Nq : 0;
+    if (o_partial_bytes) *o_partial_bytes = rows * p->d * sizeof(float);
+    if (lse_partial_bytes) *lse_partial_bytes = rows * sizeof(float);
+    return FLASH_OK;
+}
+
+FLASH_EXPORT int flash_num_splits_heuristic(int batch_nheads_mblocks, int num_SMs, int num_n_blocks, int max_splits, int seq_len)
+{
+    // Same decision procedure as src/main.cu:391-422: no split when the grid already fills four rounds of CUs;
+    // otherwise the smallest eligible split count whose last-round occupancy reaches 85 % of the best one.
+    if (num_SMs <= 0) return 1;
+    if ((float)batch_nheads_mblocks >= 4.0f * (float)num_SMs) return 1;
+    int limit = max_splits;
+    if (num_SMs < limit) limit = num_SMs;
+    if (num_n_blocks < limit) limit = num_n_blocks;
+    auto per_split = [num_n_blocks](int s) { return (num_n_blocks + s - 1) / s; };
+    auto eligible = [&](int s) {
+        return (s == 1 || per_split(s) != per_split(s - 1)) && (seq_len % (FLASH_SPLIT_KEY_GRANULE * s) == 0);
+    };
+    auto occupancy = [&](int s) {
+        const float rounds = (float)(batch_nheads_mblocks * s) / (float)num_SMs;
+        return rounds / std::ceil(rounds);
+    };
+    float best = 0.0f;
+    for (int s = 1; s <= limit; ++s)
+        if (eligible(s)) best = std::fmax(best, occupancy(s));
+    for (int s = 1; s <= limit; ++s)
+        if (eligible(s) && occupancy(s) >= 0.85 * best) return s;
+    return 1;
+}
+
+FLASH_EXPORT uint32_t flash_dropout_threshold(float dropout_p)
+{
+    double t = std::floor((double)dropout_p * 4294967296.0);
+    if (!(t > 0.0)) t = 0.0;
+    if (t > 4294967295.0) t = 4294967295.0;
+    return (uint32_t)t;
+}
+
+FLASH_EXPORT int flash_dropout_keep_mask(const flash_params* p, uint8_t* mask_out, void* stream)
+{
+    if (!p || !mask_out) return FLASH_EINVAL;
+    if (p->B < 0 || p->H < 0 || p->Nq < 0 || p->Nk < 0) return FLASH_EINVAL;
+    if (!(p->dropout_p >= 0.0f && p->dropout_p < 1.0f)) return FLASH_EINVAL;
+    if ((long long)p->B * p->H * p->Nq == 0 || p->Nk == 0) return FLASH_OK;
+    return record_hip(fa::launch_keep_mask(mask_out, p->B, p->H, p->Nq, p->Nk, flash_dropout_threshold(p->dropout_p),
+                                           p->seed, p->offset, static_cast<hipStream_t>(stream)));
+}
+
+FLASH_EXPORT const char* flash_last_hip_error(void) { return g_hip_error; }
+
+FLASH_EXPORT const char* flash_strerror(int code)
+{
+    switch (code) {
+        case FLASH_OK: return "ok";
+        case FLASH_EINVAL: return "invalid argument";
+        case FLASH_EHEADDIM: return "Insufficient shared memory. Please reduce the value of head_dim (max 128)";
+        case FLASH_EALIGN: return "pointer not aligned";
+        case FLASH_EWORKSPACE: return "split workspace missing";
+        case FLASH_ESPLITS: return "too many splits";
+        case FLASH_ELAUNCH: return "HIP launch failed";
+        case FLASH_ENODEVICE: return "no usable gfx950 device";
+        default: return "unknown error";
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,445 @@
+// Tiled FlashAttention forward for gfx950 (wave64, MFMA 32x32x16 f16 -> f32).
+//
+// Replaces forward_kernel / forward_kernel_splitkv of the reference (src/flash_forward.h:13-306,
+// src/flash_forward_splitkv.h:14-344); the math contract is the one of the reference's CPU verifier
+// (src/main.cu:309-383).  The structure is specific to CDNA4:
+//
+//  * One work-group = 4 waves; wave w owns 32*NB query rows, the group 128*NB.  KV tiles hold 64 keys.
+//  * Scores are computed transposed, S^T = K Q^T: the MFMA A operand is a K fragment read from LDS
+//    (ds_read_b128), the B operand a Q fragment that stays in registers for the whole kernel.  In the 32x32
+//    accumulator layout every lane then holds 16 keys of ONE query row (row = lane % 32), so the online-softmax
+//    max / sum are in-lane reductions plus one v_permlane32_swap between lane l and l^32.
+//  * The probabilities, rounded to fp16 where the reference rounds them (include/utils.h:47-55), already sit in
+//    the B-operand layout of O^T += V^T P^T; no LDS round trip for P.  The V^T A operand needs four keys of one
+//    head-dim column per lane: that is what ds_read_b64_tr_b16 delivers from the row-major V tile.
+//  * O^T accumulates in registers (fp32) and is normalised once in the epilogue; the reference keeps O in shared
+//    memory and renormalises it every tile (src/flash_forward.h:284-289).
+//  * K and V tiles are double-buffered in LDS; the global loads of tile t+1 are issued before the MFMA work of
+//    tile t and written to the other buffer afterwards, one barrier per tile.
+//  * Every mask of the family (causal, sliding window, key bound for ragged Nk) is one per-row interval
+//    [lo_i, hi_i] of allowed keys; tiles entirely inside the interval of every row of the wave skip the
+//    element test.  The KV tile range of the group is pruned like src/flash_forward.h:39-48.
+//  * Ragged Nq / Nk: row indices of loads are clamped, stores are predicated, keys >= Nk are masked (the
+//    reference zero-fills them and leaves them unmasked).  Head dims that are not a multiple of 8 use the
+//    element-wise load / store path (kVec = false).
+#pragma once
+#include "common.h"
+
+namespace fa {
+
+template <int D, int NB>
+struct FwdCfg {
+    static constexpr int kWaves = 4;
+    static constexpr int RW = 32 * NB;        // query rows per wave
+    static constexpr int BR = kWaves * RW;    // query rows per work-group
+    static constexpr int BC = 64;             // keys per tile
+    static constexpr int KS = D / 16;         // k-steps of the QK^T contraction
+    static constexpr int MB = D / 32;         // 32-wide head-dim blocks of O^T
+    static constexpr int CH = D / 8;          // 16-byte chunks per row
+    // LDS row strides in bytes.  K rows are read 16 bytes per lane by 32 consecutive rows: stride/16 odd spreads
+    // them over all banks.  V rows are read by ds_read_b64_tr_b16, four consecutive rows of 64 bytes per half
+    // wave: stride = 64 (mod 128) puts the four rows on disjoint bank groups.
+    static constexpr int SK = D * 2 + 16;
+    static constexpr int SV = ((D * 2) % 128 == 64) ? D * 2 : D * 2 + 64;
+    static constexpr int KBUF = BC * SK;
+    static constexpr int VBUF = BC * SV;
+    static constexpr int SMEM = 2 * KBUF + 2 * VBUF;
+    static constexpr int NLD = BC * CH / 256;  // 16-byte chunks per thread per tile (K and V each)
+    static_assert(D % 32 == 0 && D <= 128, "head-dim bucket");
+    static_assert((BC * CH) % 256 == 0, "tile chunks must divide over the group");
+};
+
+// 8 fp16 of one row starting at column col (multiple of 8); columns >= d read as zero.
+template <bool kVec>
+__device__ __forceinline__ v4u load_chunk(const half_t* __restrict__ rowp, int col, int d)
+{
+    if constexpr (kVec) {
+        const int cc = col < d ? col : d - 8;  // stay inside the row, discard below
+        v4u v = *reinterpret_cast<const v4u*>(rowp + cc);
+        const v4u z = {0u, 0u, 0u, 0u};
+        return col < d ? v : z;
+    } else {
+        union { v8h h; v4u u; } r;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int c = col + e;
+            const half_t x = rowp[c < d ? c : d - 1];
+            r.h[e] = c < d ? x : (half_t)0.0f;
+        }
+        return r.u;
+    }
+}
+
+template <int D, int NB, bool kVec, bool kAlibi, bool kDropout>
+__global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs a)
+{
+    using C = FwdCfg<D, NB>;
+    constexpr int BC = C::BC, KS = C::KS, MB = C::MB, CH = C::CH, SK = C::SK, SV = C::SV, NLD = C::NLD;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    char* const Ks = smem;
+    char* const Vs = smem + 2 * C::KBUF;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = wave_uniform(tid >> 6);
+    const int l32 = lane & 31;
+    const int g = lane >> 5;
+
+    // work-group -> (head slice, split, row block).  Slices vary fastest, so that with B*H a multiple of 8 a slice
+    // always lands on the same XCD (and L2); the heaviest causal row blocks (largest m) are dispatched first.
+    const int BH = a.B * a.H;
+    const int id = blockIdx.x;
+    const int bh = id % BH;
+    const int rest = id / BH;
+    const int split = rest % a.num_splits;
+    const int m_block = a.Tr - 1 - rest / a.num_splits;
+    const int h = bh % a.H;
+    const int Nq = a.Nq, Nk = a.Nk, d = a.d;
+    const int shift = Nk - Nq;
+    const int q0 = m_block * C::BR;
+
+    // ---- key range of the work-group (block pruning, src/flash_forward.h:39-48; split range, splitkv.h:40-43)
+    int kmin = 0, kmax = Nk;
+    {
+        const int last_row = (q0 + C::BR - 1 < Nq ? q0 + C::BR - 1 : Nq - 1) + shift;
+        if (a.wl >= 0) kmin = max(0, q0 + shift - a.wl);
+        if (a.causal) kmax = min(kmax, last_row + 1);
+        if (a.wr >= 0) kmax = min(kmax, last_row + a.wr + 1);
+        if (a.num_splits > 1) {
+            const int s0 = split * a.keys_per_split;
+            kmin = max(kmin, s0);
+            kmax = min(kmax, s0 + a.keys_per_split);
+        }
+    }
+    const int tile_begin = kmin / BC;
+    const int ntiles = kmax > kmin ? (kmax + BC - 1) / BC - tile_begin : 0;
+
+    // ---- per-lane rows
+    int row_i[NB], lo[NB], hi[NB];
+    float iif[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int i = q0 + wave * C::RW + nb * 32 + l32;
+        row_i[nb] = i;
+        const int ii = (i < Nq ? i : Nq - 1) + shift;
+        int l_ = 0, h_ = Nk - 1;
+        if (a.wl >= 0) l_ = max(0, ii - a.wl);
+        if (a.causal) h_ = min(h_, ii);
+        if (a.wr >= 0) h_ = min(h_, ii + a.wr);
+        if (a.num_splits > 1) {
+            l_ = max(l_, kmin);
+            h_ = min(h_, kmax - 1);
+        }
+        lo[nb] = l_;
+        hi[nb] = h_;
+        iif[nb] = (float)ii;
+    }
+    // wave-uniform bounds for the "does this tile need the element test" decision
+    int lo_max, hi_min;
+    {
+        const int first = q0 + wave * C::RW, last = first + C::RW - 1;
+        const int iif_ = (first < Nq ? first : Nq - 1) + shift, iil_ = (last < Nq ? last : Nq - 1) + shift;
+        lo_max = 0;
+        hi_min = Nk - 1;
+        if (a.wl >= 0) lo_max = max(0, iil_ - a.wl);
+        if (a.causal) hi_min = min(hi_min, iif_);
+        if (a.wr >= 0) hi_min = min(hi_min, iif_ + a.wr);
+        if (a.num_splits > 1) {
+            lo_max = max(lo_max, kmin);
+            hi_min = min(hi_min, kmax - 1);
+        }
+    }
+
+    const half_t* __restrict__ Qbh = a.Q + (size_t)bh * Nq * d;
+    const half_t* __restrict__ Kbh = a.K + (size_t)bh * Nk * d;
+    const half_t* __restrict__ Vbh = a.V + (size_t)bh * Nk * d;
+
+    // ---- Q fragments (B operand of S^T = K Q^T): lane holds row l32, columns 16*ks + 8*g .. +7
+    v8h qf[NB][KS];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int ic = row_i[nb] < Nq ? row_i[nb] : Nq - 1;
+        const half_t* qrow = Qbh + (size_t)ic * d;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            union { v4u u; v8h h; } t;
+            t.u = load_chunk<kVec>(qrow, 16 * ks + 8 * g, d);
+            qf[nb][ks] = t.h;
+        }
+    }
+
+    // ---- tile staging: thread handles chunk ids tid + 256*x  ->  (row, chunk) of the 64 x CH tile
+    int ld_row[NLD], ld_col[NLD];
+#pragma unroll
+    for (int x = 0; x < NLD; ++x) {
+        const int cid = tid + 256 * x;
+        ld_row[x] = cid / CH;
+        ld_col[x] = (cid % CH) * 8;
+    }
+    v4u kreg[NLD], vreg[NLD];
+    auto load_tile = [&](int tile) {
+        const int kb0 = tile * BC;
+#pragma unroll
+        for (int x = 0; x < NLD; ++x) {
+            const int r = kb0 + ld_row[x];
+            const size_t off = (size_t)(r < Nk ? r : Nk - 1) * d;
+            kreg[x] = load_chunk<kVec>(Kbh + off, ld_col[x], d);
+            vreg[x] = load_chunk<kVec>(Vbh + off, ld_col[x], d);
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int x = 0; x < NLD; ++x) {
+            *reinterpret_cast<v4u*>(Ks + buf * C::KBUF + ld_row[x] * SK + ld_col[x] * 2) = kreg[x];
+            *reinterpret_cast<v4u*>(Vs + buf * C::VBUF + ld_row[x] * SV + ld_col[x] * 2) = vreg[x];
+        }
+    };
+
+    // ---- accumulators
+    v16f oacc[MB][NB];
+    float m_run[NB], l_run[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        m_run[nb] = -INFINITY;
+        l_run[nb] = 0.0f;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[mb][nb][r] = 0.0f;
+    }
+
+    const float c2 = a.scale_log2;
+    float slope2 = 0.0f;
+    if constexpr (kAlibi) slope2 = a.alibi ? a.alibi[h] * kLog2e : 0.0f;
+
+    // LDS read offsets of this lane
+    const int k_rd = l32 * SK + g * 16;                                          // + kb*32*SK + ks*32
+    const int v_rd = (4 * g + ((lane & 15) >> 2)) * SV + (((lane >> 4) & 1) * 16 + (lane & 3) * 4) * 2;  // + row/col blocks
+
+    if (ntiles > 0) {
+        load_tile(tile_begin);
+        store_tile(0);
+    }
+    __syncthreads();
+
+    for (int t = 0; t < ntiles; ++t) {
+        const int cur = t & 1;
+        const int kb0 = (tile_begin + t) * BC;
+        const bool more = t + 1 < ntiles;
+        if (more) load_tile(tile_begin + t + 1);
+
+        // ---------------- S^T = K Q^T
+        v16f s[2][NB];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[kb][nb][r] = 0.0f;
+        const char* kbase = Ks + cur * C::KBUF + k_rd;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                const v8h af = *reinterpret_cast<const v8h*>(kbase + kb * 32 * SK + ks * 32);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                    s[kb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, qf[nb][ks], s[kb][nb], 0, 0, 0);
+            }
+        }
+
+        // ---------------- online softmax (per query row = per lane), P^T packed to fp16
+        const bool need_mask = (kb0 < lo_max) || (kb0 + BC - 1 > hi_min);
+        v8h pf[2][2][NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            if constexpr (kAlibi) {
+                // score*scale - slope*|i - j|  (src/main.cu:315,324), in the log2 domain
+                const float jb = (float)(kb0 + 4 * g) - iif[nb];
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const float dist = jb + (float)(32 * kb + 8 * (r >> 2) + (r & 3));
+                        s[kb][nb][r] = s[kb][nb][r] * c2 - slope2 * __builtin_fabsf(dist);
+                    }
+            }
+            if (need_mask) {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int j = kb0 + 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3);
+                        if (j < lo[nb] || j > hi[nb]) s[kb][nb][r] = -INFINITY;
+                    }
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kb][nb][r]);
+            mx = xhalf_max(mx);
+            if constexpr (!kAlibi) mx *= c2;  // host guarantees scale > 0 here: max commutes with the scaling
+            const float m_new = fmaxf(m_run[nb], mx);
+            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;  // fully masked so far: exp2(-inf - 0) = 0
+            const float alpha = fast_exp2(m_run[nb] - m_use);
+            m_run[nb] = m_new;
+            float rs = 0.0f;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float p;
+                    if constexpr (kAlibi) p = fast_exp2(s[kb][nb][r] - m_use);
+                    else p = fast_exp2(__builtin_fmaf(s[kb][nb][r], c2, -m_use));
+                    rs += p;
+                    s[kb][nb][r] = p;
+                }
+            l_run[nb] = l_run[nb] * alpha + rs;  // per-lane partial; halves are added in the epilogue
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0ull) {
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[mb][nb][r] *= alpha;
+            }
+            if constexpr (kDropout) {
+                // drop iff word < threshold, survivors * 1/(1-p), row sum left undropped (src/flash_forward.h:221-237)
+                const uint32_t i_u = (uint32_t)row_i[nb];
+                uint8_t* kout = a.keep_out ? a.keep_out + ((size_t)bh * Nq + row_i[nb]) * Nk : nullptr;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int rg = 0; rg < 4; ++rg) {
+                        const int j0 = kb0 + 32 * kb + 8 * rg + 4 * g;
+                        const v4u w = philox4x32_10((uint32_t)(j0 >> 2), i_u, (uint32_t)bh, a.off_lo, a.seed_lo, a.seed_hi);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const bool keep = w[e] >= a.drop_thr;
+                            s[kb][nb][4 * rg + e] = keep ? s[kb][nb][4 * rg + e] * a.drop_rscale : 0.0f;
+                            if (kout && row_i[nb] < Nq && j0 + e < Nk) kout[j0 + e] = keep ? 1 : 0;
+                        }
+                    }
+            }
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) pf[kb][tt][nb][e] = (half_t)s[kb][nb][8 * tt + e];
+        }
+
+        // ---------------- O^T += V^T P^T
+        const char* vbase = Vs + cur * C::VBUF + v_rd;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    const char* p0 = vbase + (32 * kb + 16 * tt) * SV + mb * 64;
+                    union { v4hp p[2]; v8h v; } af;
+                    af.p[0] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((FA_LDS v4hp*)(p0));
+                    af.p[1] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((FA_LDS v4hp*)(p0 + 8 * SV));
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb)
+                        oacc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af.v, pf[kb][tt][nb], oacc[mb][nb], 0, 0, 0);
+                }
+            }
+        }
+
+        if (more) store_tile(cur ^ 1);
+        __syncthreads();
+    }
+
+    // ---------------- epilogue: normalise once, store O (fp16) + LSE, or the fp32 split partials
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const float l = xhalf_sum(l_run[nb]);
+        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+        const float lse = l > 0.0f ? (m_run[nb] + fast_log2(l)) * kLn2 : -INFINITY;
+        const int i = row_i[nb];
+        if (i >= Nq) continue;
+        if (a.num_splits > 1) {
+            const size_t prow = ((size_t)bh * a.num_splits + split) * Nq + i;
+            if (g == 0) a.LSE_partial[prow] = lse;
+            float* op = a.O_partial + prow * d;
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int rg = 0; rg < 4; ++rg) {
+                    const int dc = 32 * mb + 8 * rg + 4 * g;
+                    if (kVec) {
+                        if (dc < d) {
+                            v4f o = {oacc[mb][nb][4 * rg] * inv, oacc[mb][nb][4 * rg + 1] * inv,
+                                     oacc[mb][nb][4 * rg + 2] * inv, oacc[mb][nb][4 * rg + 3] * inv};
+                            *reinterpret_cast<v4f*>(op + dc) = o;
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (dc + e < d) op[dc + e] = oacc[mb][nb][4 * rg + e] * inv;
+                    }
+                }
+        } else {
+            if (g == 0) a.LSE[(size_t)bh * Nq + i] = lse;
+            half_t* op = a.O + ((size_t)bh * Nq + i) * d;
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int rg = 0; rg < 4; ++rg) {
+                    const int dc = 32 * mb + 8 * rg + 4 * g;
+                    if (kVec) {
+                        if (dc < d) {
+                            v4h o = {(half_t)(oacc[mb][nb][4 * rg] * inv), (half_t)(oacc[mb][nb][4 * rg + 1] * inv),
+                                     (half_t)(oacc[mb][nb][4 * rg + 2] * inv), (half_t)(oacc[mb][nb][4 * rg + 3] * inv)};
+                            *reinterpret_cast<v4h*>(op + dc) = o;
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (dc + e < d) op[dc + e] = (half_t)(oacc[mb][nb][4 * rg + e] * inv);
+                    }
+                }
+        }
+    }
+}
+
+// Launcher of one head-dim bucket, defined in fwd_d{32,64,96,128}.hip.
+// variant bits: 1 = vector loads (d % 8 == 0), 2 = ALiBi, 4 = dropout.
+int launch_fwd_d32(const FwdArgs& a, int variant, int nb, hipStream_t st);
+int launch_fwd_d64(const FwdArgs& a, int variant, int nb, hipStream_t st);
+int launch_fwd_d96(const FwdArgs& a, int variant, int nb, hipStream_t st);
+int launch_fwd_d128(const FwdArgs& a, int variant, int nb, hipStream_t st);
+
+template <int D, int NB, bool kVec, bool kAlibi, bool kDropout>
+inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
+{
+    using C = FwdCfg<D, NB>;
+    auto kern = fwd_kernel<D, NB, kVec, kAlibi, kDropout>;
+    static bool attr_done = false;  // per instantiation
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    const long long groups = (long long)a.Tr * a.B * a.H * a.num_splits;
+    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(256), C::SMEM, st, a);
+    return hipGetLastError();
+}
+
+// The five instances of a bucket: vector path x {plain, ALiBi, dropout, both}; element-wise path with both features
+// compiled in (slope 0 / threshold 0 make them identities, so it serves every request with d % 8 != 0).
+template <int D, int NB>
+inline int launch_fwd_bucket(const FwdArgs& a, int variant, hipStream_t st)
+{
+    hipError_t e;
+    if (!(variant & 1)) e = launch_fwd_instance<D, NB, false, true, true>(a, st);
+    else if ((variant & 6) == 0) e = launch_fwd_instance<D, NB, true, false, false>(a, st);
+    else if ((variant & 6) == 2) e = launch_fwd_instance<D, NB, true, true, false>(a, st);
+    else if ((variant & 6) == 4) e = launch_fwd_instance<D, NB, true, false, true>(a, st);
+    else e = launch_fwd_instance<D, NB, true, true, true>(a, st);
+    return (int)e;
+}
+
+}  // namespace fa

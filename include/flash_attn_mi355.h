@@ -1,0 +1,117 @@
+/*
+ * flash_attn_mi355.h -- C ABI of the MI355X (gfx950) FlashAttention forward library.
+ *
+ * The reference (Yhorm26/flash_attn) has no host library: its interface is the kernel launch
+ *     kernel<<<dim3(Tr[*split], H, B), 256, smem>>>(mykernelParamType)
+ * issued from main() (src/main.cu:141-192) with the by-value struct of include/utils.h:21-44.
+ * The entry points below are what a binding for that path calls instead.  They take plain pointers and sizes
+ * only; every pointer in flash_params is a DEVICE pointer owned by the caller (as in src/main.cu:84-87,160-162),
+ * nothing is allocated or freed here, and work is enqueued asynchronously on the given HIP stream.
+ */
+#ifndef FLASH_ATTN_MI355_H
+#define FLASH_ATTN_MI355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Return codes.  The reference prints and exits (CUDA_CHECK, src/main.cu:18-25) or prints and returns
+ * (src/main.cu:182-185); this library returns a code instead and never terminates the process. */
+enum {
+    FLASH_OK = 0,
+    FLASH_EINVAL = -1,       /* NULL params / NULL required pointer / non-positive size / bad scalar          */
+    FLASH_EHEADDIM = -2,     /* d > 128: "Insufficient shared memory. Please reduce the value of head_dim"   */
+    FLASH_EALIGN = -3,       /* Q/K/V/O base not 16-byte aligned (reference's cp.async 16-B assumption)      */
+    FLASH_EWORKSPACE = -4,   /* num_splits > 1 but O_partial / LSE_partial missing                           */
+    FLASH_ESPLITS = -5,      /* num_splits larger than FLASH_MAX_SPLITS                                      */
+    FLASH_ELAUNCH = -6,      /* the HIP runtime rejected a launch; see flash_last_hip_error()                */
+    FLASH_ENODEVICE = -7     /* no gfx950 device / code object not loadable on the current device           */
+};
+
+#define FLASH_MAX_HEAD_DIM 128
+#define FLASH_MAX_SPLITS 128
+#define FLASH_SPLIT_KEY_GRANULE 128 /* key-block size the split ranges are cut at (reference Bc, main.cu:117) */
+
+/* Superset of mykernelParamType (include/utils.h:21-44).
+ *   reference field            here
+ *   Q,K,V (half*)              Q,K,V            fp16 [B,H,Nq|Nk,d] contiguous, same layout
+ *   O (float*)                 O                fp16 [B,H,Nq,d]  (the reference stores fp32)
+ *   --                         LSE              fp32 [B,H,Nq]    natural-log sum-exp of the masked scaled scores
+ *   O_tmp, L, M                O_partial, LSE_partial   fp32 [B,H,S,Nq,d] and [B,H,S,Nq]; LSE_s = M_s + log L_s
+ *   N, d (+ gridDim.y/.z)      B, H, Nq, Nk, d
+ *   Br,Bc,Tr,Tc                not part of the ABI (tiling is the library's business)
+ *   softmax_scale              softmax_scale
+ *   window_size_left/right     window_left/right   (< 0: unbounded on that side; reference uses -1 for "off")
+ *   --                         is_causal           (template bool Is_causal in the reference)
+ *   alibi_slopes_ptr           alibi_slopes        fp32 [H] or NULL; score -= slope[h] * |i - j|
+ *   dropout_prob, seed, states dropout_p, seed, offset   counter-based Philox4x32-10 instead of curand states
+ *   split_num                  num_splits          (<= 0: flash_num_splits_heuristic with 256 CUs)
+ * Row index used by masks and bias is i + (Nk - Nq), which is i whenever Nq == Nk (all the reference can express).
+ */
+typedef struct flash_params {
+    const void *Q;
+    const void *K;
+    const void *V;
+    void *O;
+    float *LSE;
+    float *O_partial;
+    float *LSE_partial;
+    int B, H, Nq, Nk, d;
+    float softmax_scale;
+    int is_causal;
+    int window_left;
+    int window_right;
+    const float *alibi_slopes;
+    float dropout_p;
+    uint64_t seed;
+    uint64_t offset;
+    int num_splits;
+    /* Optional debug output: when non-NULL and dropout_p > 0, the forward kernel also stores the keep decision it
+     * applied to every in-range (i, j) as one byte (1 = kept) into keep_mask_out [B,H,Nq,Nk].  No counterpart in
+     * the reference, whose dropout is never verified (src/main.cu:44,222). */
+    uint8_t *keep_mask_out;
+} flash_params;
+
+/* Tiled forward over the whole key range: replaces
+ *     forward_kernel<...><<<dim3(Tr,H,B),256,smem>>>(param)              (src/flash_forward.h:13-15, src/main.cu:189)
+ * `stream` is a hipStream_t passed as void* (NULL = default stream, which is what the reference uses). */
+int flash_forward(const flash_params *p, void *stream);
+
+/* Split-KV forward plus combine on the same stream: replaces
+ *     forward_kernel_splitkv<...><<<dim3(Tr*split,H,B),256,smem>>>(param);
+ *     forward_kernel_splitkv_combine<<<dim3(Tr,H,B),Br>>>(param);          (src/flash_forward_splitkv.h:14-16,347-348,
+ *                                                                          src/main.cu:189-192)
+ * Uses p->num_splits (heuristic when <= 0); needs the workspace when the resulting split count is > 1. */
+int flash_forward_splitkv(const flash_params *p, void *stream);
+
+/* Bytes of O_partial and of LSE_partial needed for p (the cudaMallocs of src/main.cu:160-162). Either may be NULL. */
+int flash_splitkv_workspace_bytes(const flash_params *p, size_t *o_partial_bytes, size_t *lse_partial_bytes);
+
+/* The split count flash_forward_splitkv will use for p (after the heuristic and clamping). */
+int flash_splitkv_resolve_splits(const flash_params *p);
+
+/* num_splits_heuristic (src/main.cu:391-422), same arguments and return value; main() passes num_SMs = 108,
+ * this library's callers pass the CU count (256). */
+int flash_num_splits_heuristic(int batch_nheads_mblocks, int num_SMs, int num_n_blocks, int max_splits, int seq_len);
+
+/* Keep-mask of the dropout contract alone, [B,H,Nq,Nk] bytes on the device (uses B,H,Nq,Nk,dropout_p,seed,offset of
+ * p).  Stands where init_curand_states<<<...>>> (src/init_curand_states.h:7-14, src/main.cu:128-139) stood as the
+ * separately launched RNG step; the counter-based generator needs no state, so this only materialises the mask. */
+int flash_dropout_keep_mask(const flash_params *p, uint8_t *mask_out, void *stream);
+
+/* Integer drop threshold floor(p * 2^32) (host helper; element kept iff its Philox word >= threshold). */
+uint32_t flash_dropout_threshold(float dropout_p);
+
+/* Text of the last HIP error seen by this thread inside the library ("" if none). */
+const char *flash_last_hip_error(void);
+
+/* Human-readable name of a return code. */
+const char *flash_strerror(int code);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASH_ATTN_MI355_H */
