@@ -1,0 +1,252 @@
+#!/usr/bin/env python3
+"""Benchmark of the FlashAttention-forward hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only-main]
+
+A step is one pass of the hot path over one batch of synthetic input already resident in HBM.  The headline
+workload is the causal prefill configuration (B=4, H=16, Nq=Nk=2048, d=128); the split-KV decode configuration
+(B=16, H=32, Nq=1, Nk=16384, d=128, 16 splits) and the remaining configurations are timed beside it and reported
+in extra keys of the same JSON line.  Timing protocol: warm-up launches, then K back-to-back launches between two
+HIP events on the launch stream (the reference's protocol, src/main.cu:187-213), plus a host clock around the same
+region for ms_per_step.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_F16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
+PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E
+METRIC = "fwd attention TFLOP/s + % fp16 MFMA peak; split-KV decode HBM GB/s"
+
+
+def unmasked_pairs(Nq, Nk, causal, wl, wr):
+    """Number of (i, j) pairs a head attends to (row index i + Nk - Nq)."""
+    shift = Nk - Nq
+    total = 0
+    for i in range(Nq):
+        ii = i + shift
+        lo = max(0, ii - wl) if wl >= 0 else 0
+        hi = Nk - 1
+        if causal:
+            hi = min(hi, ii)
+        if wr >= 0:
+            hi = min(hi, ii + wr)
+        total += max(0, hi - lo + 1)
+    return total
+
+
+CONFIGS = {
+    "cfg1": dict(B=1, H=2, Nq=128, Nk=128, d=64, causal=False, window=(-1, -1), alibi=False, p=0.0, splits=0),
+    "cfg2": dict(B=4, H=16, Nq=2048, Nk=2048, d=128, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=0),
+    "cfg3": dict(B=2, H=16, Nq=4096, Nk=4096, d=64, causal=False, window=(256, 0), alibi=True, p=0.0, splits=0),
+    "cfg4": dict(B=8, H=32, Nq=1000, Nk=1000, d=96, causal=True, window=(-1, -1), alibi=False, p=0.1, splits=0),
+    "cfg5": dict(B=16, H=32, Nq=1, Nk=16384, d=128, causal=False, window=(-1, -1), alibi=False, p=0.0, splits=16),
+}
+# diagnostic shapes (not part of the contract; selectable with --workload, never in the default line)
+DIAG = {
+    "diag_noncausal": dict(B=4, H=16, Nq=2048, Nk=2048, d=128, causal=False, window=(-1, -1), alibi=False, p=0.0, splits=0),
+    "diag_d64": dict(B=4, H=16, Nq=2048, Nk=2048, d=64, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=0),
+    "diag_long": dict(B=1, H=16, Nq=8192, Nk=8192, d=128, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=0),
+}
+DESCR = {
+    "cfg1": "plain fwd B=1 H=2 Nq=Nk=128 d=64",
+    "cfg2": "causal prefill fwd B=4 H=16 Nq=Nk=2048 d=128",
+    "cfg3": "local(256,0)+ALiBi fwd B=2 H=16 Nq=Nk=4096 d=64",
+    "cfg4": "causal+dropout(0.1) fwd B=8 H=32 Nq=Nk=1000 d=96",
+    "cfg5": "split-KV decode B=16 H=32 Nq=1 Nk=16384 d=128 num_splits=16",
+    "diag_noncausal": "non-causal fwd B=4 H=16 Nq=Nk=2048 d=128 (diagnostic)",
+    "diag_d64": "causal fwd B=4 H=16 Nq=Nk=2048 d=64 (diagnostic)",
+    "diag_long": "causal fwd B=1 H=16 Nq=Nk=8192 d=128 (diagnostic)",
+}
+
+
+def flops_of(c):
+    P = unmasked_pairs(c["Nq"], c["Nk"], c["causal"], *c["window"])
+    return 4.0 * c["d"] * c["B"] * c["H"] * P
+
+
+def decode_bytes(c):
+    kv = 2 * c["B"] * c["H"] * c["Nk"] * c["d"] * 2
+    q = c["B"] * c["H"] * c["Nq"] * c["d"] * 2
+    o = c["B"] * c["H"] * c["Nq"] * c["d"] * 2
+    lse = c["B"] * c["H"] * c["Nq"] * 4
+    return kv + q + o + lse
+
+
+def make_inputs(c, seed=0):
+    import torch
+
+    g = torch.Generator(device="cuda")
+    out = []
+    for n, s in ((c["Nq"], 1), (c["Nk"], 2), (c["Nk"], 3)):
+        g.manual_seed(3 * seed + s)
+        out.append(torch.randn((c["B"], c["H"], n, c["d"]), generator=g, device="cuda", dtype=torch.float32).half())
+    return out
+
+
+def make_step(fa, c, q, k, v):
+    """Returns a zero-argument callable that enqueues one pass (no allocation inside)."""
+    import ctypes as C
+    import torch
+    from flash_attn_amd import binding
+
+    B, H, Nq, Nk, d = c["B"], c["H"], c["Nq"], c["Nk"], c["d"]
+    o = torch.empty((B, H, Nq, d), dtype=torch.float16, device="cuda")
+    lse = torch.empty((B, H, Nq), dtype=torch.float32, device="cuda")
+    slopes = None
+    if c["alibi"]:
+        slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / H) for h in range(H)], dtype=torch.float32, device="cuda")
+    ws = (None, None)
+    if c["splits"]:
+        S = fa.resolve_splits(B, H, Nq, Nk, d, c["splits"])
+        if S > 1:
+            ws = (torch.empty((B, H, S, Nq, d), dtype=torch.float32, device="cuda"),
+                  torch.empty((B, H, S, Nq), dtype=torch.float32, device="cuda"))
+    p = binding.make_params(q, k, v, o, lse, None, c["causal"], c["window"], slopes, c["p"], 1234, 0,
+                            c["splits"] if c["splits"] else 1, ws[0], ws[1])
+    lib = fa.lib()
+    fn = lib.flash_forward_splitkv if c["splits"] else lib.flash_forward
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    keep = (q, k, v, o, lse, slopes, ws)
+
+    def step():
+        rc = fn(C.byref(p), stream)
+        if rc != 0:
+            raise RuntimeError(f"launch failed: {rc} {keep is None}")
+
+    return step, (o, lse)
+
+
+def time_steps(step, steps, warmup):
+    """(host ms per step, event ms per step) over `steps` back-to-back launches."""
+    import torch
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+
+
+def cpu_baseline(c, q, k, v, budget_slices):
+    """The reference's own attention_forward_cpu (oracle/_ref, compiled from the reference checkout) on a bounded
+    sample of (b,h) slices, one core as in the reference; falls back to the restatement when _ref is absent."""
+    import numpy as np
+    from oracle import cpu_oracle as co
+
+    n = max(1, min(budget_slices, c["B"] * c["H"]))
+    H = c["H"]
+    # slices 0..n-1 of batch entry 0 (n <= H)
+    n = min(n, H)
+    qs = q[0:1, :n].float().cpu().numpy()
+    ks = k[0:1, :n].float().cpu().numpy()
+    vs = v[0:1, :n].float().cpu().numpy()
+    scale = 1.0 / math.sqrt(c["d"])
+    P = unmasked_pairs(c["Nq"], c["Nk"], c["causal"], *c["window"])
+    fl = 4.0 * c["d"] * n * P
+    if co.ref_lib() is not None and c["Nq"] == c["Nk"]:
+        t0 = time.perf_counter()
+        co.ref_attention_forward_cpu(qs, ks, vs, scale, causal=c["causal"])
+        dt = time.perf_counter() - t0
+        kind = "reference"
+    else:
+        t0 = time.perf_counter()
+        co.attention_forward(qs, ks, vs, scale, causal=c["causal"], nthreads=1, skip_masked=False)
+        dt = time.perf_counter() - t0
+        kind = "port"
+    return {"value": fl / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": kind,
+            "sample": f"{n} of {c['B'] * c['H']} (b,h) slices of the same workload, {dt:.2f} s, "
+                      f"algorithmic flops of the sample / time"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--only-main", action="store_true", help="time only the headline workload (for profiling)")
+    ap.add_argument("--workload", default="cfg2", choices=sorted(CONFIGS) + sorted(DIAG), help="headline workload")
+    ap.add_argument("--cpu-slices", type=int, default=16)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no multi-GPU path exists); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import flash_attn_amd as fa
+
+    fa.lib()  # fails loudly when the HIP library is missing
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+
+    name = args.workload
+    c = CONFIGS[name] if name in CONFIGS else DIAG[name]
+    q, k, v = make_inputs(c)
+    step, _ = make_step(fa, c, q, k, v)
+    host_ms, ev_ms = time_steps(step, args.steps, args.warmup)
+    if name == "cfg5":
+        by = decode_bytes(c)
+        value, unit = by / (host_ms * 1e-3) / 1e9, "GB/s"
+        roof = {"bound": "hbm", "achieved": by / (ev_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBPS, "unit": "GB/s"}
+    else:
+        fl = flops_of(c)
+        value, unit = fl / (host_ms * 1e-3) / 1e12, "TFLOP/s"
+        roof = {"bound": "mfma", "achieved": fl / (ev_ms * 1e-3) / 1e12, "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = None
+    roof["kernel_ms"] = ev_ms
+
+    result = {
+        "metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": host_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic", "config": {"workload": f"{name}: {DESCR[name]}", "inputs": "fp16 RN(N(0,1)), seeded, resident in HBM",
+                                        "accumulate": "fp32", "outputs": "fp16 O + fp32 LSE"},
+        "roofline": roof,
+    }
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(c, q, k, v, args.cpu_slices)
+    del q, k, v, step
+
+    if not args.only_main:
+        others = {}
+        for n2, c2 in CONFIGS.items():
+            if n2 == name:
+                continue
+            q, k, v = make_inputs(c2)
+            st, _ = make_step(fa, c2, q, k, v)
+            steps2 = 1000 if n2 == "cfg1" else 100
+            _, ev = time_steps(st, steps2, 5)
+            if n2 == "cfg5":
+                by = decode_bytes(c2)
+                others[n2] = {"workload": DESCR[n2], "ms": ev, "GB/s": by / (ev * 1e-3) / 1e9,
+                              "frac_hbm_peak": by / (ev * 1e-3) / 1e9 / PEAK_HBM_GBPS, "algorithmic_bytes": by}
+            else:
+                fl = flops_of(c2)
+                others[n2] = {"workload": DESCR[n2], "ms": ev, "TFLOP/s": fl / (ev * 1e-3) / 1e12,
+                              "frac_mfma_peak": fl / (ev * 1e-3) / 1e12 / PEAK_F16_TFLOPS, "algorithmic_flops": fl}
+            del q, k, v, st
+        result["other_workloads"] = others
+        if "cfg5" in others:
+            result["roofline_decode"] = {"bound": "hbm", "achieved": others["cfg5"]["GB/s"], "peak": PEAK_HBM_GBPS,
+                                         "unit": "GB/s", "frac": others["cfg5"]["frac_hbm_peak"], "traffic": None}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -45,15 +45,19 @@ struct FwdCfg {
     static constexpr int VBUF = BC * SV;
     static constexpr int SMEM = 2 * KBUF + 2 * VBUF;
     static constexpr int NLD = BC * CH / 256;  // 16-byte chunks per thread per tile (K and V each)
+    static constexpr bool kPipelined = false;  // issue S(t+1) = K(t+1) Q^T next to softmax(S(t)); costs 32*NB registers
     static_assert(D % 32 == 0 && D <= 128, "head-dim bucket");
     static_assert((BC * CH) % 256 == 0, "tile chunks must divide over the group");
 };
 
 // 8 fp16 of one row starting at column col (multiple of 8); columns >= d read as zero.
-template <bool kVec>
+// kVec: rows are 16-byte aligned (d % 8 == 0); kFullD: d equals the bucket width, no column test at all.
+template <bool kVec, bool kFullD>
 __device__ __forceinline__ v4u load_chunk(const half_t* __restrict__ rowp, int col, int d)
 {
-    if constexpr (kVec) {
+    if constexpr (kFullD) {
+        return *reinterpret_cast<const v4u*>(rowp + col);
+    } else if constexpr (kVec) {
         const int cc = col < d ? col : d - 8;  // stay inside the row, discard below
         v4u v = *reinterpret_cast<const v4u*>(rowp + cc);
         const v4u z = {0u, 0u, 0u, 0u};
@@ -70,9 +74,19 @@ __device__ __forceinline__ v4u load_chunk(const half_t* __restrict__ rowp, int c
     }
 }
 
-template <int D, int NB, bool kVec, bool kAlibi, bool kDropout>
+// Running maximum is only raised when some row of the wave outgrows it by more than this many powers of two;
+// until then probabilities are taken relative to the stale maximum (bounded by 2^kLazyTau, exact in the end
+// because numerator and denominator carry the same factor).  Saves the per-tile rescale of the O accumulators.
+constexpr float kLazyTau = 8.0f;
+
+// variant bits of the kernel template
+constexpr int kVarVec = 1, kVarAlibi = 2, kVarDropout = 4, kVarFullD = 8;
+
+template <int D, int NB, int VAR>
 __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs a)
 {
+    constexpr bool kVec = (VAR & kVarVec) != 0, kAlibi = (VAR & kVarAlibi) != 0, kDropout = (VAR & kVarDropout) != 0,
+                   kFullD = (VAR & kVarFullD) != 0;
     using C = FwdCfg<D, NB>;
     constexpr int BC = C::BC, KS = C::KS, MB = C::MB, CH = C::CH, SK = C::SK, SV = C::SV, NLD = C::NLD;
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -94,7 +108,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
     const int split = rest % a.num_splits;
     const int m_block = a.Tr - 1 - rest / a.num_splits;
     const int h = bh % a.H;
-    const int Nq = a.Nq, Nk = a.Nk, d = a.d;
+    const int Nq = a.Nq, Nk = a.Nk, d = kFullD ? D : a.d;
     const int shift = Nk - Nq;
     const int q0 = m_block * C::BR;
 
@@ -163,7 +177,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             union { v4u u; v8h h; } t;
-            t.u = load_chunk<kVec>(qrow, 16 * ks + 8 * g, d);
+            t.u = load_chunk<kVec, kFullD>(qrow, 16 * ks + 8 * g, d);
             qf[nb][ks] = t.h;
         }
     }
@@ -177,30 +191,31 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
         ld_col[x] = (cid % CH) * 8;
     }
     v4u kreg[NLD], vreg[NLD];
-    auto load_tile = [&](int tile) {
+    auto gload = [&](const half_t* __restrict__ base, int tile, v4u (&reg)[NLD]) {
         const int kb0 = tile * BC;
 #pragma unroll
         for (int x = 0; x < NLD; ++x) {
             const int r = kb0 + ld_row[x];
-            const size_t off = (size_t)(r < Nk ? r : Nk - 1) * d;
-            kreg[x] = load_chunk<kVec>(Kbh + off, ld_col[x], d);
-            vreg[x] = load_chunk<kVec>(Vbh + off, ld_col[x], d);
+            reg[x] = load_chunk<kVec, kFullD>(base + (size_t)(r < Nk ? r : Nk - 1) * d, ld_col[x], d);
         }
     };
-    auto store_tile = [&](int buf) {
+    auto put_k = [&](int buf) {
 #pragma unroll
-        for (int x = 0; x < NLD; ++x) {
+        for (int x = 0; x < NLD; ++x)
             *reinterpret_cast<v4u*>(Ks + buf * C::KBUF + ld_row[x] * SK + ld_col[x] * 2) = kreg[x];
+    };
+    auto put_v = [&](int buf) {
+#pragma unroll
+        for (int x = 0; x < NLD; ++x)
             *reinterpret_cast<v4u*>(Vs + buf * C::VBUF + ld_row[x] * SV + ld_col[x] * 2) = vreg[x];
-        }
     };
 
     // ---- accumulators
     v16f oacc[MB][NB];
-    float m_run[NB], l_run[NB];
+    float m_ref[NB], l_run[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-        m_run[nb] = -INFINITY;
+        m_ref[nb] = -INFINITY;
         l_run[nb] = 0.0f;
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
@@ -216,27 +231,15 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
     const int k_rd = l32 * SK + g * 16;                                          // + kb*32*SK + ks*32
     const int v_rd = (4 * g + ((lane & 15) >> 2)) * SV + (((lane >> 4) & 1) * 16 + (lane & 3) * 4) * 2;  // + row/col blocks
 
-    if (ntiles > 0) {
-        load_tile(tile_begin);
-        store_tile(0);
-    }
-    __syncthreads();
-
-    for (int t = 0; t < ntiles; ++t) {
-        const int cur = t & 1;
-        const int kb0 = (tile_begin + t) * BC;
-        const bool more = t + 1 < ntiles;
-        if (more) load_tile(tile_begin + t + 1);
-
-        // ---------------- S^T = K Q^T
-        v16f s[2][NB];
+    // S^T = K Q^T of the tile in K buffer `buf`
+    auto qk = [&](int buf, v16f (&s)[2][NB]) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s[kb][nb][r] = 0.0f;
-        const char* kbase = Ks + cur * C::KBUF + k_rd;
+        const char* kbase = Ks + buf * C::KBUF + k_rd;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
@@ -247,10 +250,10 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
                     s[kb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, qf[nb][ks], s[kb][nb], 0, 0, 0);
             }
         }
+    };
 
-        // ---------------- online softmax (per query row = per lane), P^T packed to fp16
-        const bool need_mask = (kb0 < lo_max) || (kb0 + BC - 1 > hi_min);
-        v8h pf[2][2][NB];
+    // online softmax of one tile (per query row = per lane); leaves P^T packed to fp16 in pf
+    auto softmax = [&](bool need_mask, int kb0, v16f (&s)[2][NB], v8h (&pf)[2][2][NB]) {
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             if constexpr (kAlibi) {
@@ -265,12 +268,16 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
                     }
             }
             if (need_mask) {
+                // wave-uniform and rare (boundary tiles only).  Routing the bounds through an empty volatile asm keeps
+                // this a real branch: otherwise the compiler folds the block into selects that every tile executes.
+                int lo_rel = lo[nb] - kb0 - 4 * g, hi_rel = hi[nb] - kb0 - 4 * g;
+                asm volatile("; boundary tile: element mask" : "+v"(lo_rel), "+v"(hi_rel));
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        const int j = kb0 + 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3);
-                        if (j < lo[nb] || j > hi[nb]) s[kb][nb][r] = -INFINITY;
+                        const int jr = 32 * kb + 8 * (r >> 2) + (r & 3);
+                        if (jr < lo_rel || jr > hi_rel) s[kb][nb][r] = -INFINITY;
                     }
             }
             float mx = -INFINITY;
@@ -280,10 +287,18 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
                 for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kb][nb][r]);
             mx = xhalf_max(mx);
             if constexpr (!kAlibi) mx *= c2;  // host guarantees scale > 0 here: max commutes with the scaling
-            const float m_new = fmaxf(m_run[nb], mx);
-            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;  // fully masked so far: exp2(-inf - 0) = 0
-            const float alpha = fast_exp2(m_run[nb] - m_use);
-            m_run[nb] = m_new;
+            if (__builtin_amdgcn_ballot_w64(mx > m_ref[nb] + kLazyTau) != 0ull) {
+                const float m_new = fmaxf(m_ref[nb], mx);
+                float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_ref[nb] - m_new);
+                asm volatile("; raise running max" : "+v"(alpha));  // keeps the rescale inside this rare branch
+                m_ref[nb] = m_new;
+                l_run[nb] *= alpha;
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[mb][nb][r] *= alpha;
+            }
+            const float m_use = (m_ref[nb] == -INFINITY) ? 0.0f : m_ref[nb];  // nothing seen yet: exp2(-inf - 0) = 0
             float rs = 0.0f;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
@@ -295,13 +310,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
                     rs += p;
                     s[kb][nb][r] = p;
                 }
-            l_run[nb] = l_run[nb] * alpha + rs;  // per-lane partial; halves are added in the epilogue
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0ull) {
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[mb][nb][r] *= alpha;
-            }
+            l_run[nb] += rs;  // per-lane partial; the two half-waves are added in the epilogue
             if constexpr (kDropout) {
                 // drop iff word < threshold, survivors * 1/(1-p), row sum left undropped (src/flash_forward.h:221-237)
                 const uint32_t i_u = (uint32_t)row_i[nb];
@@ -327,9 +336,11 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
 #pragma unroll
                     for (int e = 0; e < 8; ++e) pf[kb][tt][nb][e] = (half_t)s[kb][nb][8 * tt + e];
         }
+    };
 
-        // ---------------- O^T += V^T P^T
-        const char* vbase = Vs + cur * C::VBUF + v_rd;
+    // O^T += V^T P^T with the tile in V buffer `buf`
+    auto pv = [&](int buf, v8h (&pf)[2][2][NB]) {
+        const char* vbase = Vs + buf * C::VBUF + v_rd;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
@@ -346,9 +357,88 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
                 }
             }
         }
+    };
 
-        if (more) store_tile(cur ^ 1);
+    // The Q fragments must have landed before the loop starts: a load still counted as outstanding at the loop
+    // header makes the compiler guard every use of qf inside the loop with a vmcnt wait, and since vmcnt counts in
+    // order, that wait would also drain the K/V prefetch of the same iteration.
+    auto pin_q = [&]() {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[nb][ks]));
+    };
+
+    if constexpr (!C::kPipelined) {
+        // ---- plain double-buffered loop: tile t+1 is fetched from global memory while tile t is computed.
+        if (ntiles > 0) {
+            gload(Kbh, tile_begin, kreg);
+            gload(Vbh, tile_begin, vreg);
+            put_k(0);
+            put_v(0);
+        }
+        pin_q();
         __syncthreads();
+        for (int t = 0; t < ntiles; ++t) {
+            const int cur = t & 1;
+            const int kb0 = (tile_begin + t) * BC;
+            const bool has1 = t + 1 < ntiles;
+            if (has1) {
+                gload(Kbh, tile_begin + t + 1, kreg);
+                gload(Vbh, tile_begin + t + 1, vreg);
+            }
+            v16f s[2][NB];
+            v8h pf[2][2][NB];
+            qk(cur, s);
+            const bool need_mask = (kb0 < lo_max) || (kb0 + BC - 1 > hi_min);
+            softmax(need_mask, kb0, s, pf);
+            pv(cur, pf);
+            if (has1) {
+                put_k(cur ^ 1);
+                put_v(cur ^ 1);
+            }
+            __syncthreads();
+        }
+    } else {
+        // ---- software pipeline.  Iteration t works on tile t: S(t) was produced one iteration earlier, so the
+        // MFMAs of S(t+1) = K(t+1) Q^T are issued next to the VALU work of softmax(S(t)), followed by O += P(t) V(t).
+        // LDS: K(t+1) in K buffer (t+1)&1, V(t) in V buffer t&1; the global loads of K(t+2) and V(t+1) fly meanwhile
+        // and are written to the freed buffers before the single barrier of the iteration.
+        v16f s_cur[2][NB];
+        if (ntiles > 0) {
+            gload(Kbh, tile_begin, kreg);
+            gload(Vbh, tile_begin, vreg);
+            put_k(0);
+            put_v(0);
+            if (ntiles > 1) {
+                gload(Kbh, tile_begin + 1, kreg);
+                put_k(1);
+            }
+        }
+        pin_q();
+        __syncthreads();
+        if (ntiles > 0) qk(0, s_cur);
+        for (int t = 0; t < ntiles; ++t) {
+            const int kb0 = (tile_begin + t) * BC;
+            const bool has1 = t + 1 < ntiles, has2 = t + 2 < ntiles;
+            if (has2) gload(Kbh, tile_begin + t + 2, kreg);
+            if (has1) gload(Vbh, tile_begin + t + 1, vreg);
+            const bool need_mask = (kb0 < lo_max) || (kb0 + BC - 1 > hi_min);
+            v8h pf[2][2][NB];
+            v16f s_next[2][NB];
+            if (has1) qk((t + 1) & 1, s_next);
+            softmax(need_mask, kb0, s_cur, pf);
+            pv(t & 1, pf);
+            if (has2) put_k(t & 1);
+            if (has1) put_v((t + 1) & 1);
+            __syncthreads();
+            if (has1) {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) s_cur[kb][nb] = s_next[kb][nb];
+            }
+        }
     }
 
     // ---------------- epilogue: normalise once, store O (fp16) + LSE, or the fp32 split partials
@@ -356,7 +446,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
     for (int nb = 0; nb < NB; ++nb) {
         const float l = xhalf_sum(l_run[nb]);
         const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-        const float lse = l > 0.0f ? (m_run[nb] + fast_log2(l)) * kLn2 : -INFINITY;
+        const float lse = l > 0.0f ? (m_ref[nb] + fast_log2(l)) * kLn2 : -INFINITY;
         const int i = row_i[nb];
         if (i >= Nq) continue;
         if (a.num_splits > 1) {
@@ -369,7 +459,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
                 for (int rg = 0; rg < 4; ++rg) {
                     const int dc = 32 * mb + 8 * rg + 4 * g;
                     if (kVec) {
-                        if (dc < d) {
+                        if (kFullD || dc < d) {
                             v4f o = {oacc[mb][nb][4 * rg] * inv, oacc[mb][nb][4 * rg + 1] * inv,
                                      oacc[mb][nb][4 * rg + 2] * inv, oacc[mb][nb][4 * rg + 3] * inv};
                             *reinterpret_cast<v4f*>(op + dc) = o;
@@ -389,7 +479,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
                 for (int rg = 0; rg < 4; ++rg) {
                     const int dc = 32 * mb + 8 * rg + 4 * g;
                     if (kVec) {
-                        if (dc < d) {
+                        if (kFullD || dc < d) {
                             v4h o = {(half_t)(oacc[mb][nb][4 * rg] * inv), (half_t)(oacc[mb][nb][4 * rg + 1] * inv),
                                      (half_t)(oacc[mb][nb][4 * rg + 2] * inv), (half_t)(oacc[mb][nb][4 * rg + 3] * inv)};
                             *reinterpret_cast<v4h*>(op + dc) = o;
@@ -405,17 +495,17 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
 }
 
 // Launcher of one head-dim bucket, defined in fwd_d{32,64,96,128}.hip.
-// variant bits: 1 = vector loads (d % 8 == 0), 2 = ALiBi, 4 = dropout.
+// variant bits: kVarVec (d % 8 == 0), kVarAlibi, kVarDropout; kVarFullD is derived here (d == bucket width).
 int launch_fwd_d32(const FwdArgs& a, int variant, int nb, hipStream_t st);
 int launch_fwd_d64(const FwdArgs& a, int variant, int nb, hipStream_t st);
 int launch_fwd_d96(const FwdArgs& a, int variant, int nb, hipStream_t st);
 int launch_fwd_d128(const FwdArgs& a, int variant, int nb, hipStream_t st);
 
-template <int D, int NB, bool kVec, bool kAlibi, bool kDropout>
+template <int D, int NB, int VAR>
 inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
 {
     using C = FwdCfg<D, NB>;
-    auto kern = fwd_kernel<D, NB, kVec, kAlibi, kDropout>;
+    auto kern = fwd_kernel<D, NB, VAR>;
     static bool attr_done = false;  // per instantiation
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -428,17 +518,27 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
     return hipGetLastError();
 }
 
-// The five instances of a bucket: vector path x {plain, ALiBi, dropout, both}; element-wise path with both features
-// compiled in (slope 0 / threshold 0 make them identities, so it serves every request with d % 8 != 0).
+// The nine instances of a bucket: {d == bucket, d % 8 == 0} x {plain, ALiBi, dropout, both}, and the element-wise
+// path with both features compiled in (slope 0 / threshold 0 make them identities, so it serves every request
+// with d % 8 != 0).
 template <int D, int NB>
 inline int launch_fwd_bucket(const FwdArgs& a, int variant, hipStream_t st)
 {
     hipError_t e;
-    if (!(variant & 1)) e = launch_fwd_instance<D, NB, false, true, true>(a, st);
-    else if ((variant & 6) == 0) e = launch_fwd_instance<D, NB, true, false, false>(a, st);
-    else if ((variant & 6) == 2) e = launch_fwd_instance<D, NB, true, true, false>(a, st);
-    else if ((variant & 6) == 4) e = launch_fwd_instance<D, NB, true, false, true>(a, st);
-    else e = launch_fwd_instance<D, NB, true, true, true>(a, st);
+    const int feat = variant & (kVarAlibi | kVarDropout);
+    if (!(variant & kVarVec)) {
+        e = launch_fwd_instance<D, NB, kVarAlibi | kVarDropout>(a, st);
+    } else if (a.d == D) {
+        if (feat == 0) e = launch_fwd_instance<D, NB, kVarVec | kVarFullD>(a, st);
+        else if (feat == kVarAlibi) e = launch_fwd_instance<D, NB, kVarVec | kVarFullD | kVarAlibi>(a, st);
+        else if (feat == kVarDropout) e = launch_fwd_instance<D, NB, kVarVec | kVarFullD | kVarDropout>(a, st);
+        else e = launch_fwd_instance<D, NB, kVarVec | kVarFullD | kVarAlibi | kVarDropout>(a, st);
+    } else {
+        if (feat == 0) e = launch_fwd_instance<D, NB, kVarVec>(a, st);
+        else if (feat == kVarAlibi) e = launch_fwd_instance<D, NB, kVarVec | kVarAlibi>(a, st);
+        else if (feat == kVarDropout) e = launch_fwd_instance<D, NB, kVarVec | kVarDropout>(a, st);
+        else e = launch_fwd_instance<D, NB, kVarVec | kVarAlibi | kVarDropout>(a, st);
+    }
     return (int)e;
 }
 

@@ -1,0 +1,143 @@
+"""CPU tests of the boundary: the shared library loads, exports every symbol the public header declares, its struct
+matches the header, argument checking returns codes without touching a GPU, and the host-side logic (split
+heuristic, split resolution, workspace sizing, dropout threshold) agrees with the oracle / golden tables."""
+import ctypes as C
+import json
+import os
+import re
+import subprocess
+import tempfile
+
+import numpy as np
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+HEADER = os.path.join(ROOT, "include", "flash_attn_mi355.h")
+
+E_INVAL, E_HEADDIM, E_ALIGN, E_WORKSPACE, E_SPLITS = -1, -2, -3, -4, -5
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(flash_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(fa):
+    names = declared_functions()
+    assert {"flash_forward", "flash_forward_splitkv", "flash_splitkv_workspace_bytes",
+            "flash_num_splits_heuristic", "flash_dropout_keep_mask"} <= set(names)
+    L = C.CDLL(fa.library_path())
+    for n in names:
+        assert hasattr(L, n), f"{n} declared in the header but not exported"
+
+
+def test_ctypes_struct_matches_header(fa):
+    """sizeof / offsetof from the C compiler against the ctypes mirror."""
+    fields = [f[0] for f in fa.FlashParams._fields_]
+    prog = "#include <stdio.h>\n#include <stddef.h>\n#include \"flash_attn_mi355.h\"\nint main(){printf(\"%zu\\n\",sizeof(flash_params));\n"
+    for f in fields:
+        prog += f'printf("%zu\\n", offsetof(flash_params, {f}));\n'
+    prog += "return 0;}\n"
+    with tempfile.TemporaryDirectory() as td:
+        src, exe = os.path.join(td, "t.c"), os.path.join(td, "t")
+        open(src, "w").write(prog)
+        subprocess.check_call(["gcc", "-std=c99", "-I", os.path.join(ROOT, "include"), src, "-o", exe])
+        out = [int(x) for x in subprocess.check_output([exe]).split()]
+    assert out[0] == C.sizeof(fa.FlashParams)
+    for f, off in zip(fields, out[1:]):
+        assert getattr(fa.FlashParams, f).offset == off, f
+
+
+def _params(fa, **kw):
+    p = fa.FlashParams()
+    p.B, p.H, p.Nq, p.Nk, p.d = 1, 1, 16, 16, 64
+    p.softmax_scale = 0.125
+    p.window_left = p.window_right = -1
+    p.num_splits = 1
+    # fake but well-aligned device addresses: validation must reject before anything is dereferenced or launched
+    p.Q, p.K, p.V, p.O, p.LSE = 0x1000, 0x2000, 0x3000, 0x4000, 0x5000
+    for k, v in kw.items():
+        setattr(p, k, v)
+    return p
+
+
+def test_argument_errors_are_codes_not_aborts(fa):
+    L = fa.lib()
+    assert L.flash_forward(None, None) == E_INVAL
+    assert L.flash_forward_splitkv(None, None) == E_INVAL
+    for entry in (L.flash_forward, L.flash_forward_splitkv):
+        assert entry(C.byref(_params(fa, d=0)), None) == E_INVAL
+        assert entry(C.byref(_params(fa, d=-4)), None) == E_INVAL
+        assert entry(C.byref(_params(fa, Nq=-1)), None) == E_INVAL
+        assert entry(C.byref(_params(fa, d=129)), None) == E_HEADDIM  # reference: "Please reduce the value of head_dim"
+        assert entry(C.byref(_params(fa, d=256)), None) == E_HEADDIM
+        assert entry(C.byref(_params(fa, Q=None)), None) == E_INVAL
+        assert entry(C.byref(_params(fa, O=None)), None) == E_INVAL
+        assert entry(C.byref(_params(fa, LSE=None)), None) == E_INVAL
+        assert entry(C.byref(_params(fa, K=None)), None) == E_INVAL
+        assert entry(C.byref(_params(fa, Q=0x1008)), None) == E_ALIGN
+        assert entry(C.byref(_params(fa, V=0x3002)), None) == E_ALIGN
+        assert entry(C.byref(_params(fa, dropout_p=1.0)), None) == E_INVAL
+        assert entry(C.byref(_params(fa, dropout_p=-0.1)), None) == E_INVAL
+        assert entry(C.byref(_params(fa, dropout_p=float("nan"))), None) == E_INVAL
+        assert entry(C.byref(_params(fa, softmax_scale=float("inf"))), None) == E_INVAL
+        assert entry(C.byref(_params(fa, num_splits=129)), None) == E_SPLITS
+        # empty problems are a no-op
+        assert entry(C.byref(_params(fa, B=0)), None) == 0
+        assert entry(C.byref(_params(fa, Nq=0, Q=None, O=None, LSE=None)), None) == 0
+    # a split run without its workspace
+    assert L.flash_forward_splitkv(C.byref(_params(fa, Nk=1024, num_splits=4)), None) == E_WORKSPACE
+    # odd head dims only need element alignment
+    assert L.flash_forward(C.byref(_params(fa, d=31, Q=0x1001)), None) == E_ALIGN
+    for code in (0, -1, -2, -3, -4, -5, -6, -7):
+        assert L.flash_strerror(code)
+    assert b"head_dim" in L.flash_strerror(E_HEADDIM)
+
+
+def test_heuristic_matches_reference_table(fa, oracle):
+    t = json.load(open(os.path.join(HERE, "golden", "heuristic_table.json")))
+    for *args, want in t["rows"]:
+        assert fa.num_splits_heuristic(*args) == want, args
+    rng = np.random.default_rng(0)
+    for _ in range(2000):
+        nblk = int(rng.integers(1, 200))
+        args = (int(rng.integers(1, 3000)), int(rng.choice([108, 256, 64])), nblk, int(rng.integers(1, 200)),
+                nblk * 128 if rng.random() < 0.8 else int(rng.integers(1, 30000)))
+        assert fa.num_splits_heuristic(*args) == oracle.num_splits_heuristic(*args), args
+
+
+def test_split_resolution_and_workspace(fa):
+    # decode configuration: caller pins 16 splits
+    assert fa.resolve_splits(16, 32, 1, 16384, 128, 16) == 16
+    assert fa.workspace_bytes(16, 32, 1, 16384, 128, 16) == (16 * 32 * 16 * 1 * 128 * 4, 16 * 32 * 16 * 4)
+    # never more splits than 128-key blocks; one split needs no workspace
+    assert fa.resolve_splits(1, 1, 1, 300, 64, 16) == 3
+    assert fa.resolve_splits(1, 1, 128, 128, 64, 8) == 1
+    assert fa.workspace_bytes(1, 1, 128, 128, 64, 8) == (0, 0)
+    # heuristic (num_splits <= 0) with 256 CUs: the reference's checked-in shape B=1,H=8,N=1021 splits 4 ways,
+    # every benchmark shape stays unsplit
+    assert fa.resolve_splits(1, 8, 1021, 1021, 31, 0) == 4
+    assert fa.resolve_splits(4, 16, 2048, 2048, 128, 0) == 1
+    assert fa.resolve_splits(16, 32, 1, 16384, 128, 0) == 1
+    with pytest.raises(fa.FlashError):
+        fa.resolve_splits(1, 1, 1, 128, 64, 1000)
+
+
+def test_dropout_threshold_matches_oracle(fa, oracle):
+    for p in (0.0, 0.1, 0.25, 0.5, 0.3333, 0.9, 0.999999):
+        assert fa.dropout_threshold(p) == oracle.dropout_threshold(p)
+
+
+def test_product_does_not_reach_into_the_oracle():
+    pkg = os.path.join(ROOT, "flash_attn_amd")
+    for dirpath, _, files in os.walk(pkg):
+        if "build" in dirpath:
+            continue
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp", "Makefile")):
+                text = open(os.path.join(dirpath, f), errors="ignore").read()
+                assert "oracle" not in text, f"{f} mentions the oracle"
+    out = subprocess.check_output(["nm", "-D", os.path.join(pkg, "lib", "libflash_attn_mi355.so")]).decode()
+    assert "oracle_" not in out

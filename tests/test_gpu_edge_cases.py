@@ -1,0 +1,203 @@
+"""GPU parity on the edge cases of the path: ragged sizes, odd head dims, Nq != Nk, window / ALiBi / causal combinations,
+fully masked rows, dropout determinism, general split-KV (Nq > 1) with every mask, empty problems, and size-independent
+properties at full size.  Everything goes through the C ABI; the checker is the CPU oracle."""
+import numpy as np
+import pytest
+
+from helpers import check_o_lse, oracle_forward_batched, randn_f16_gpu, to_f32_np
+
+pytestmark = pytest.mark.gpu
+
+
+def _qkv(B, H, Nq, Nk, d, seed=0):
+    return (randn_f16_gpu((B, H, Nq, d), 3 * seed + 1), randn_f16_gpu((B, H, Nk, d), 3 * seed + 2),
+            randn_f16_gpu((B, H, Nk, d), 3 * seed + 3))
+
+
+def _slopes(oracle, H):
+    import torch
+    s = oracle.alibi_slopes(H)
+    return s, torch.from_numpy(s).cuda()
+
+
+# head dims: every bucket edge, multiples of 8 that are not bucket widths, and odd values (element-wise path);
+# 31 is the reference's checked-in head_dim (src/main.cu:42)
+@pytest.mark.parametrize("d", [8, 16, 24, 31, 32, 33, 40, 64, 72, 96, 100, 127, 128])
+def test_head_dims(fa, oracle, d):
+    q, k, v = _qkv(2, 3, 150, 150, d, seed=d)
+    for kw in (dict(), dict(causal=True)):
+        o, lse = fa.flash_forward(q, k, v, **kw)
+        O, L = oracle_forward_batched(oracle, q, k, v, **kw)
+        check_o_lse(o, lse, O, L, f"d={d} {kw}")
+
+
+# sequence lengths around the tile sizes (64-key tiles, 128-row groups); 1021 is the reference's checked-in seq_len
+@pytest.mark.parametrize("N", [1, 2, 31, 63, 64, 65, 127, 128, 129, 191, 257, 1000, 1021])
+def test_ragged_lengths(fa, oracle, N):
+    q, k, v = _qkv(1, 2, N, N, 64, seed=N)
+    sl, sl_t = _slopes(oracle, 2)
+    for kw, okw in ((dict(), dict()), (dict(causal=True), dict(causal=True)),
+                    (dict(window=(37, 5), alibi_slopes=sl_t), dict(window=(37, 5), slopes=sl))):
+        o, lse = fa.flash_forward(q, k, v, **kw)
+        O, L = oracle_forward_batched(oracle, q, k, v, **okw)
+        check_o_lse(o, lse, O, L, f"N={N} {list(kw)}")
+
+
+@pytest.mark.parametrize("Nq,Nk", [(1, 700), (5, 333), (64, 1000), (200, 77), (130, 131), (300, 64)])
+def test_nq_differs_from_nk(fa, oracle, Nq, Nk):
+    """Mask and bias row index is i + Nk - Nq.  Nk < Nq with a causal mask leaves leading rows with nothing to attend
+    to: O = 0 and LSE = -inf there."""
+    q, k, v = _qkv(2, 2, Nq, Nk, 64, seed=Nq + Nk)
+    sl, sl_t = _slopes(oracle, 2)
+    for kw, okw in ((dict(), dict()), (dict(causal=True), dict(causal=True)),
+                    (dict(window=(50, 10)), dict(window=(50, 10))),
+                    (dict(causal=True, alibi_slopes=sl_t), dict(causal=True, slopes=sl))):
+        o, lse = fa.flash_forward(q, k, v, **kw)
+        O, L = oracle_forward_batched(oracle, q, k, v, **okw)
+        check_o_lse(o, lse, O, L, f"Nq={Nq} Nk={Nk} {list(kw)}")
+
+
+@pytest.mark.parametrize("window", [(0, 0), (1, 0), (0, 3), (100, 100), (128, 128), (256, 0), (5, 300), (-1, 7), (9, -1)])
+def test_windows(fa, oracle, window):
+    """window (128,128) is the reference's own window_attention setting (src/main.cu:57-60)."""
+    q, k, v = _qkv(1, 2, 520, 520, 64, seed=11)
+    o, lse = fa.flash_forward(q, k, v, window=window)
+    O, L = oracle_forward_batched(oracle, q, k, v, window=window)
+    check_o_lse(o, lse, O, L, f"window={window}")
+    o, lse = fa.flash_forward(q, k, v, window=window, causal=True)
+    O, L = oracle_forward_batched(oracle, q, k, v, window=window, causal=True)
+    check_o_lse(o, lse, O, L, f"window={window} causal")
+
+
+def test_alibi_all_buckets(fa, oracle):
+    for d in (32, 64, 96, 128, 48):
+        H = 4
+        q, k, v = _qkv(1, H, 300, 300, d, seed=d + 1)
+        sl, sl_t = _slopes(oracle, H)
+        o, lse = fa.flash_forward(q, k, v, alibi_slopes=sl_t, causal=True)
+        O, L = oracle_forward_batched(oracle, q, k, v, slopes=sl, causal=True)
+        check_o_lse(o, lse, O, L, f"alibi d={d}")
+
+
+def test_scale_values(fa, oracle):
+    """A non-positive scale takes the kernel variant that scales before the row maximum."""
+    q, k, v = _qkv(1, 2, 200, 200, 64, seed=5)
+    for scale in (1.0, 0.02, -0.125, 0.0):
+        o, lse = fa.flash_forward(q, k, v, softmax_scale=scale, causal=True)
+        O, L = oracle_forward_batched(oracle, q, k, v, scale=scale, causal=True)
+        check_o_lse(o, lse, O, L, f"scale={scale}")
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 200, 200, 64), (1, 2, 100, 333, 96), (1, 2, 129, 129, 31), (1, 1, 300, 300, 128)])
+def test_dropout_mask_bit_exact_and_output(fa, oracle, shape):
+    import torch
+    B, H, Nq, Nk, d = shape
+    q, k, v = _qkv(B, H, Nq, Nk, d, seed=sum(shape))
+    for p, seed, off in ((0.1, 1234, 0), (0.5, 2 ** 40 + 17, 3), (0.9, 7, 2 ** 33 + 5)):
+        o, lse, km = fa.flash_forward(q, k, v, dropout_p=p, seed=seed, offset=off, return_keep_mask=True)
+        keep = oracle.dropout_keep_mask(seed, off, p, B, H, Nq, Nk)
+        assert np.array_equal(km.cpu().numpy(), keep), "fused kernel's keep decisions differ from the CPU Philox replica"
+        assert np.array_equal(fa.dropout_keep_mask(B, H, Nq, Nk, p, seed, off).cpu().numpy(), keep)
+        O, L = oracle_forward_batched(oracle, q, k, v, keep_mask=torch.from_numpy(keep), p_drop=p)
+        check_o_lse(o, lse, O, L, f"dropout p={p} {shape}")
+        # same seed, same result; the mask does not depend on whether it is dumped
+        o2, _ = fa.flash_forward(q, k, v, dropout_p=p, seed=seed, offset=off)
+        assert torch.equal(o, o2)
+
+
+@pytest.mark.parametrize("S", [1, 2, 3, 5, 8])
+def test_general_splitkv_matches_unsplit(fa, oracle, S):
+    """The reference's split path for Nq > 1 (its checked-in run: N=1021, d=31, src/main.cu:39-49) with every mask;
+    result must not depend on the split count, and the partials must match the oracle's restatement."""
+    B, H, N, d = 1, 4, 1021, 31
+    q, k, v = _qkv(B, H, N, N, d, seed=S)
+    sl, sl_t = _slopes(oracle, H)
+    for kw, okw in ((dict(), dict()), (dict(causal=True), dict(causal=True)),
+                    (dict(window=(300, 40), alibi_slopes=sl_t), dict(window=(300, 40), slopes=sl))):
+        o, lse, ws = fa.flash_forward_splitkv(q, k, v, num_splits=S, return_partials=True, **kw)
+        O, L = oracle_forward_batched(oracle, q, k, v, **okw)
+        check_o_lse(o, lse, O, L, f"split S={S} {list(kw)}")
+        if S > 1:
+            Ot, Ls, Ms, LSEp = oracle.splitkv_partials(to_f32_np(q), to_f32_np(k), to_f32_np(v), S, **okw)
+            op, lp = to_f32_np(ws[0]), to_f32_np(ws[1])
+            assert np.array_equal(np.isneginf(lp), np.isneginf(LSEp))
+            fin = np.isfinite(LSEp)
+            assert np.abs(lp[fin] - LSEp[fin]).max() <= 1e-4
+            assert np.abs(op - Ot).max() <= 2e-3
+
+
+def test_splitkv_heuristic_and_decode_variants(fa, oracle):
+    # num_splits <= 0: the library's heuristic (4 splits for this shape on 256 CUs)
+    q, k, v = _qkv(1, 8, 1021, 1021, 32, seed=3)
+    o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=0)
+    O, L = oracle_forward_batched(oracle, q, k, v)
+    check_o_lse(o, lse, O, L, "heuristic split")
+    # decode kernel: head-dim buckets, ragged Nk, window, ALiBi, one split and many
+    for d, Nk, S in ((128, 5000, 7), (64, 777, 3), (32, 130, 2), (96, 4096, 16), (128, 300, 1), (40, 1000, 4)):
+        H = 4
+        q, k, v = _qkv(2, H, 1, Nk, d, seed=d + Nk)
+        sl, sl_t = _slopes(oracle, H)
+        for kw, okw in ((dict(), dict()), (dict(window=(200, 0), alibi_slopes=sl_t), dict(window=(200, 0), slopes=sl)),
+                        (dict(causal=True), dict(causal=True))):
+            o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=S, **kw)
+            O, L = oracle_forward_batched(oracle, q, k, v, **okw)
+            check_o_lse(o, lse, O, L, f"decode d={d} Nk={Nk} S={S} {list(kw)}")
+    # Nq == 1 with an odd head dim or dropout falls back to the tiled kernel
+    q, k, v = _qkv(1, 2, 1, 900, 31, seed=9)
+    o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=4)
+    O, L = oracle_forward_batched(oracle, q, k, v)
+    check_o_lse(o, lse, O, L, "decode odd d")
+
+
+def test_empty_and_degenerate(fa):
+    import torch
+    z = lambda *s: torch.zeros(s, dtype=torch.float16, device="cuda")
+    o, lse = fa.flash_forward(z(0, 2, 16, 64), z(0, 2, 16, 64), z(0, 2, 16, 64))
+    assert o.shape == (0, 2, 16, 64)
+    o, lse = fa.flash_forward(z(1, 2, 0, 64), z(1, 2, 16, 64), z(1, 2, 16, 64))
+    assert o.shape == (1, 2, 0, 64)
+    # no keys at all: every row is fully masked
+    o, lse = fa.flash_forward(randn_f16_gpu((1, 2, 10, 64), 1), z(1, 2, 0, 64), z(1, 2, 0, 64))
+    assert torch.all(o == 0) and torch.all(torch.isneginf(lse))
+    o, lse = fa.flash_forward_splitkv(randn_f16_gpu((1, 2, 1, 64), 1), z(1, 2, 0, 64), z(1, 2, 0, 64), num_splits=4)
+    assert torch.all(o == 0) and torch.all(torch.isneginf(lse))
+
+
+def test_head_dim_limit_is_an_error(fa):
+    import torch
+    t = torch.zeros((1, 1, 16, 136), dtype=torch.float16, device="cuda")
+    with pytest.raises(fa.FlashError) as e:
+        fa.flash_forward(t, t, t)
+    assert e.value.code == -2
+
+
+def test_full_size_properties_causal_prefill(fa):
+    """Size-independent checks at the full benchmark shape (B=4,H=16,N=2048,d=128): V = const gives O = const;
+    permuting the heads permutes the result; LSE of row 0 is the single score it sees."""
+    import torch
+    B, H, N, d = 4, 16, 2048, 128
+    q, k, v = _qkv(B, H, N, N, d, seed=77)
+    ones = torch.ones_like(v)
+    o, lse = fa.flash_forward(q, k, ones, causal=True)
+    assert torch.allclose(o.float(), torch.ones_like(o, dtype=torch.float32), atol=2e-3)
+    o1, l1 = fa.flash_forward(q, k, v, causal=True)
+    perm = torch.randperm(H, device="cuda")
+    o2, l2 = fa.flash_forward(q[:, perm].contiguous(), k[:, perm].contiguous(), v[:, perm].contiguous(), causal=True)
+    assert torch.equal(o1[:, perm], o2) and torch.equal(l1[:, perm], l2)
+    s00 = (q[:, :, 0].float() * k[:, :, 0].float()).sum(-1) * d ** -0.5
+    assert torch.allclose(l1[:, :, 0], s00, atol=1e-4)
+    assert torch.allclose(o1[:, :, 0].float(), v[:, :, 0].float(), atol=2e-3, rtol=1e-2)
+
+
+def test_full_size_properties_decode(fa):
+    """Decode shape (B=16,H=32,Nk=16384,d=128): independence of the split count and the V = const identity."""
+    import torch
+    B, H, Nk, d = 16, 32, 16384, 128
+    q, k, v = _qkv(B, H, 1, Nk, d, seed=78)
+    o16, l16 = fa.flash_forward_splitkv(q, k, v, num_splits=16)
+    for S in (1, 4, 128):
+        oS, lS = fa.flash_forward_splitkv(q, k, v, num_splits=S)
+        assert torch.allclose(oS.float(), o16.float(), atol=1e-3)
+        assert torch.allclose(lS, l16, atol=2e-5)
+    o, _ = fa.flash_forward_splitkv(q, k, torch.full_like(v, 0.5), num_splits=16)
+    assert torch.allclose(o.float(), torch.full_like(o, 0.5, dtype=torch.float32), atol=1e-3)

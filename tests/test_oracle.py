@@ -1,0 +1,250 @@
+"""CPU tests that pin the oracle (oracle/attention_oracle.c): golden vectors written from the reference's own
+compiled CPU functions, the live compiled reference where oracle/_ref exists, float64 brute force, closed forms
+and invariants.  None of these needs a GPU."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+GOLD = os.path.join(HERE, "golden")
+
+
+def brute(q, k, v, scale, causal=False, wl=-1, wr=-1, slopes=None, keep=None, p=0.0):
+    """Independent float64 formulation on the full score matrix. Returns O, LSE."""
+    q, k, v = [np.asarray(a, dtype=np.float64) for a in (q, k, v)]
+    B, H, Nq, d = q.shape
+    Nk = k.shape[2]
+    s = np.einsum("bhid,bhjd->bhij", q, k) * float(scale)
+    ii = np.arange(Nq)[:, None] + (Nk - Nq)
+    jj = np.arange(Nk)[None, :]
+    if slopes is not None:
+        s = s - np.asarray(slopes, dtype=np.float64)[None, :, None, None] * np.abs(ii - jj)[None, None]
+    mask = np.zeros((Nq, Nk), dtype=bool)
+    if causal:
+        mask |= jj > ii
+    if wl >= 0:
+        mask |= (ii - jj) > wl
+    if wr >= 0:
+        mask |= (jj - ii) > wr
+    s = np.where(mask[None, None], -np.inf, s)
+    m = s.max(axis=-1, keepdims=True)
+    msafe = np.where(np.isfinite(m), m, 0.0)
+    e = np.exp(s - msafe)
+    l = e.sum(axis=-1, keepdims=True)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        pmat = np.where(l > 0, e / l, 0.0)
+        lse = np.where(l[..., 0] > 0, msafe[..., 0] + np.log(l[..., 0]), -np.inf)
+    if keep is not None:
+        pmat = np.where(keep.astype(bool), pmat / (1.0 - p), 0.0)
+    return np.einsum("bhij,bhjd->bhid", pmat, v), lse
+
+
+def rand_qkv(rng, B, H, Nq, Nk, d):
+    f = lambda *s: rng.standard_normal(s).astype(np.float16).astype(np.float32)
+    return f(B, H, Nq, d), f(B, H, Nk, d), f(B, H, Nk, d)
+
+
+# ---------------------------------------------------------------------------------------------- golden vectors
+def test_golden_reference_vectors_bit_exact(oracle):
+    g = np.load(os.path.join(GOLD, "reference_cpu_vectors.npz"))
+    cases = {"A": ["plain", "causal"], "B": ["plain", "causal", "window9", "alibi", "causal_alibi_window20"]}
+    kw = {"plain": {}, "causal": dict(causal=True), "window9": dict(window=(9, 9)), "alibi": dict(use_slopes=True),
+          "causal_alibi_window20": dict(causal=True, window=(20, 20), use_slopes=True)}
+    for tag, names in cases.items():
+        q, k, v = [g[f"{tag}_{n}"].astype(np.float32) for n in "qkv"]
+        for name in names:
+            a = dict(kw[name])
+            slopes = g[f"{tag}_slopes"] if a.pop("use_slopes", False) else None
+            for skip in (True, False):
+                O, _ = oracle.attention_forward(q, k, v, float(g[f"{tag}_scale"]), slopes=slopes, skip_masked=skip,
+                                                nthreads=2, **a)
+                assert np.array_equal(O, g[f"{tag}_O_{name}"]), (tag, name, skip)
+
+
+def test_golden_heuristic_table(oracle):
+    t = json.load(open(os.path.join(GOLD, "heuristic_table.json")))
+    for *args, want in t["rows"]:
+        assert oracle.num_splits_heuristic(*args) == want, args
+
+
+def test_golden_verfiy_counts(oracle):
+    for c in json.load(open(os.path.join(GOLD, "verfiy_cases.json"))):
+        dev = np.array([float(x) for x in c["dev"]], dtype=np.float32)
+        assert oracle.verify_count(np.array(c["cpu"], dtype=np.float32), dev, c["tol"]) == c["count"]
+
+
+# ------------------------------------------------------------------------- live compiled reference (this container)
+def test_live_reference_bit_exact(oracle):
+    if oracle.ref_lib() is None:
+        pytest.skip("oracle/_ref not built (reference checkout absent)")
+    rng = np.random.default_rng(3)
+    for (B, H, N, d) in [(1, 2, 128, 64), (2, 3, 50, 31), (1, 1, 257, 96), (1, 4, 33, 128)]:
+        q, k, v = rand_qkv(rng, B, H, N, N, d)
+        # the reference's own input distribution too: U(0,10), unrounded fp32 (src/main.cu:91-97)
+        qu, ku, vu = [rng.uniform(0, 10, size=(B, H, N, d)).astype(np.float32) for _ in range(3)]
+        sl = oracle.alibi_slopes(H)
+        scale = np.float32(1.0 / np.sqrt(d))
+        for (a, b, c) in ((q, k, v), (qu, ku, vu)):
+            for causal, w, s in [(False, -1, None), (True, -1, None), (False, 7, None), (False, -1, sl), (True, 16, sl),
+                                 (False, 0, None)]:
+                R = oracle.ref_attention_forward_cpu(a, b, c, scale, causal=causal, window_size=w, slopes=s)
+                O, _ = oracle.attention_forward(a, b, c, scale, causal=causal, window=(w, w), slopes=s, nthreads=2)
+                assert np.array_equal(O, R), (B, H, N, d, causal, w, s is not None)
+    for args in [(64, 108, 8, 8, 1024), (64, 256, 8, 8, 1024), (3, 256, 5, 5, 640), (512, 256, 128, 128, 16384)]:
+        assert oracle.num_splits_heuristic(*args) == oracle.ref_num_splits_heuristic(*args)
+
+
+# ------------------------------------------------------------------------------------------ brute force / closed forms
+@pytest.mark.parametrize("shape", [(1, 2, 8, 8, 4), (2, 2, 17, 17, 24), (1, 3, 5, 29, 16), (1, 1, 40, 13, 8), (1, 2, 1, 300, 32)])
+def test_brute_force_all_features(oracle, shape):
+    B, H, Nq, Nk, d = shape
+    rng = np.random.default_rng(sum(shape))
+    q, k, v = rand_qkv(rng, B, H, Nq, Nk, d)
+    sl = oracle.alibi_slopes(H)
+    scale = 1.0 / np.sqrt(d)
+    for causal, (wl, wr), s in [(False, (-1, -1), None), (True, (-1, -1), None), (False, (3, 0), None), (False, (0, 5), None),
+                                (False, (2, 7), sl), (True, (4, -1), sl), (False, (-1, 2), None)]:
+        O, L = oracle.attention_forward(q, k, v, scale, causal=causal, window=(wl, wr), slopes=s, nthreads=2)
+        Ob, Lb = brute(q, k, v, scale, causal, wl, wr, s)
+        assert np.abs(O - Ob).max() < 2e-5, (shape, causal, wl, wr)
+        assert np.array_equal(np.isneginf(L), np.isneginf(Lb))
+        fin = np.isfinite(Lb)
+        assert np.abs(L[fin] - Lb[fin]).max() < 2e-5
+        # fully masked rows: O = 0, LSE = -inf
+        assert np.all(O[~fin] == 0.0)
+
+
+def test_lse_normalises_scores(oracle):
+    rng = np.random.default_rng(11)
+    q, k, v = rand_qkv(rng, 1, 2, 33, 65, 16)
+    scale = 0.25
+    _, L = oracle.attention_forward(q, k, v, scale)
+    s = np.einsum("bhid,bhjd->bhij", q.astype(np.float64), k.astype(np.float64)) * scale
+    assert np.abs(np.exp(s - L[..., None].astype(np.float64)).sum(-1) - 1.0).max() < 1e-5
+
+
+def test_unbounded_left_zero_right_is_causal(oracle):
+    rng = np.random.default_rng(12)
+    q, k, v = rand_qkv(rng, 1, 2, 70, 70, 32)
+    Oc, Lc = oracle.attention_forward(q, k, v, causal=True)
+    Ow, Lw = oracle.attention_forward(q, k, v, window=(-1, 0))
+    assert np.array_equal(Oc, Ow) and np.array_equal(Lc, Lw)
+
+
+def test_skip_masked_is_bit_identical(oracle):
+    rng = np.random.default_rng(13)
+    q, k, v = rand_qkv(rng, 1, 2, 90, 90, 40)
+    sl = oracle.alibi_slopes(2)
+    for kw in (dict(causal=True), dict(window=(5, 9), slopes=sl), dict(window=(200, 0))):
+        a = oracle.attention_forward(q, k, v, skip_masked=True, **kw)
+        b = oracle.attention_forward(q, k, v, skip_masked=False, **kw)
+        assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+
+
+def test_zero_padding_with_key_bound_equals_unpadded(oracle):
+    """Tail contract: padding N and d with zeros changes nothing once keys >= Nk are masked (here: not present)."""
+    rng = np.random.default_rng(14)
+    q, k, v = rand_qkv(rng, 1, 2, 37, 37, 24)
+    O, L = oracle.attention_forward(q, k, v, scale=0.2, causal=True)
+    qp, kp, vp = [np.pad(a, ((0, 0), (0, 0), (0, 0), (0, 8))) for a in (q, k, v)]
+    Op, Lp = oracle.attention_forward(qp, kp, vp, scale=0.2, causal=True)
+    assert np.abs(Op[..., :24] - O).max() < 1e-6 and np.all(Op[..., 24:] == 0) and np.abs(L - Lp).max() < 1e-6
+
+
+def test_alibi_slopes_closed_form(oracle):
+    for H in (1, 2, 8, 16, 32):
+        want = np.array([2.0 ** (-8.0 * (h + 1) / H) for h in range(H)])
+        assert np.abs(oracle.alibi_slopes(H) - want).max() < 1e-7
+
+
+# --------------------------------------------------------------------------------------------------------- dropout
+def test_philox_known_answers(oracle):
+    # Random123 kat_vectors, philox4x32 10 rounds
+    assert oracle.philox4x32_10([0, 0, 0, 0], [0, 0]) == [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]
+    assert oracle.philox4x32_10([0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2) == [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]
+    assert oracle.philox4x32_10([0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0]) == [
+        0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]
+
+
+def test_philox_against_independent_python(oracle):
+    def py_philox(ctr, key):
+        c, k = list(ctr), list(key)
+        for _ in range(10):
+            p0, p1 = 0xD2511F53 * c[0], 0xCD9E8D57 * c[2]
+            c = [((p1 >> 32) ^ c[1] ^ k[0]) & 0xFFFFFFFF, p1 & 0xFFFFFFFF, ((p0 >> 32) ^ c[3] ^ k[1]) & 0xFFFFFFFF,
+                 p0 & 0xFFFFFFFF]
+            k = [(k[0] + 0x9E3779B9) & 0xFFFFFFFF, (k[1] + 0xBB67AE85) & 0xFFFFFFFF]
+        return c
+    rng = np.random.default_rng(1)
+    for _ in range(50):
+        ctr = [int(x) for x in rng.integers(0, 2 ** 32, 4)]
+        key = [int(x) for x in rng.integers(0, 2 ** 32, 2)]
+        assert oracle.philox4x32_10(ctr, key) == py_philox(ctr, key)
+
+
+def test_dropout_threshold_and_mask_layout(oracle):
+    assert oracle.dropout_threshold(0.0) == 0
+    assert oracle.dropout_threshold(0.5) == 2 ** 31
+    assert oracle.dropout_threshold(0.25) == 2 ** 30
+    assert oracle.dropout_threshold(0.1) == int(np.floor(float(np.float32(0.1)) * 2 ** 32))
+    B, H, Nq, Nk, p = 2, 3, 5, 11, 0.3
+    seed, off = 0x1234567812345678, 9
+    m = oracle.dropout_keep_mask(seed, off, p, B, H, Nq, Nk)
+    thr = oracle.dropout_threshold(p)
+    for (b, h, i, j) in [(0, 0, 0, 0), (1, 2, 4, 10), (0, 1, 3, 7), (1, 0, 2, 5)]:
+        w = oracle.philox4x32_10([j >> 2, i, b * H + h, off], [seed & 0xFFFFFFFF, seed >> 32])[j & 3]
+        assert m[b, h, i, j] == (1 if w >= thr else 0)
+    assert oracle.dropout_keep_mask(1, 0, 0.0, 1, 1, 4, 9).all()
+    big = oracle.dropout_keep_mask(1234, 0, 0.1, 1, 4, 256, 256)
+    assert abs(big.mean() - 0.9) < 0.005
+    assert not np.array_equal(big, oracle.dropout_keep_mask(1235, 0, 0.1, 1, 4, 256, 256))
+    assert not np.array_equal(big, oracle.dropout_keep_mask(1234, 1, 0.1, 1, 4, 256, 256))
+
+
+def test_dropout_semantics(oracle):
+    rng = np.random.default_rng(21)
+    q, k, v = rand_qkv(rng, 1, 2, 19, 23, 16)
+    O0, L0 = oracle.attention_forward(q, k, v, causal=True)
+    ones = np.ones((1, 2, 19, 23), dtype=np.uint8)
+    O1, L1 = oracle.attention_forward(q, k, v, causal=True, keep_mask=ones, p_drop=0.0)
+    assert np.array_equal(O0, O1) and np.array_equal(L0, L1)
+    keep = oracle.dropout_keep_mask(7, 0, 0.4, 1, 2, 19, 23)
+    O2, L2 = oracle.attention_forward(q, k, v, causal=True, keep_mask=keep, p_drop=0.4)
+    Ob, Lb = brute(q, k, v, 1 / np.sqrt(16), causal=True, keep=keep, p=float(np.float32(0.4)))
+    assert np.abs(O2 - Ob).max() < 2e-5
+    assert np.array_equal(L2, L0)  # the row sum stays undropped
+
+
+# --------------------------------------------------------------------------------------------------------- split-KV
+def test_split_ranges_partition_keys(oracle):
+    for Nk in (1, 127, 128, 129, 1000, 1021, 16384):
+        for S in (1, 2, 3, 8, 16):
+            r = [oracle.split_key_range(Nk, S, s) for s in range(S)]
+            assert r[0][0] == 0 and r[-1][1] == Nk
+            for a, b in zip(r, r[1:]):
+                assert a[1] == b[0]
+            assert all(a[0] % 128 == 0 for a in r if a[0] < Nk)
+    assert oracle.split_key_range(16384, 16, 3) == (3072, 4096)
+
+
+@pytest.mark.parametrize("S", [1, 2, 3, 8, 16])
+def test_split_combine_equals_unsplit(oracle, S):
+    rng = np.random.default_rng(30 + S)
+    B, H, Nq, Nk, d = 1, 2, 9, 1021, 31
+    q, k, v = rand_qkv(rng, B, H, Nq, Nk, d)
+    sl = oracle.alibi_slopes(H)
+    for kw in (dict(), dict(causal=True), dict(window=(300, 40), slopes=sl)):
+        O, L = oracle.attention_forward(q, k, v, **kw)
+        Ot, Ls, Ms, LSEp = oracle.splitkv_partials(q, k, v, S, **kw)
+        Oc, Lc = oracle.splitkv_combine(Ot, Ls, Ms)
+        assert np.abs(Oc - O).max() < 1e-5
+        assert np.abs(Lc - L).max() < 1e-5
+        # the LSE form of the workspace carries the same information: LSE = logsumexp_s LSE_s
+        with np.errstate(divide="ignore"):
+            mx = LSEp.max(axis=2, keepdims=True)
+            lse2 = (mx + np.log(np.exp(LSEp - mx).sum(axis=2, keepdims=True)))[:, :, 0]
+            w = np.exp(LSEp - lse2[:, :, None])
+        assert np.abs(lse2 - L).max() < 1e-5
+        assert np.abs((w[..., None] * Ot).sum(axis=2) - O).max() < 1e-5
