@@ -66,6 +66,22 @@ DESCR = {
 }
 
 
+PROFILE_OF = {"cfg2": "fwd_kernel_d128_causal_prefill.md", "cfg5": "decode_split_kernel_d128_splitkv_decode.md"}
+
+
+def measured_traffic(name):
+    """HBM bytes per launch from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary of this workload (the line
+    `traffic_bytes_per_launch: N` of the file under profiles/), or None when no summary exists."""
+    f = PROFILE_OF.get(name)
+    path = os.path.join(ROOT, "profiles", f) if f else None
+    if not path or not os.path.exists(path):
+        return None
+    for line in open(path):
+        if line.startswith("traffic_bytes_per_launch:"):
+            return float(line.split(":")[1])
+    return None
+
+
 def flops_of(c):
     P = unmasked_pairs(c["Nq"], c["Nk"], c["causal"], *c["window"])
     return 4.0 * c["d"] * c["B"] * c["H"] * P
@@ -181,6 +197,9 @@ def main():
     ap.add_argument("--only-main", action="store_true", help="time only the headline workload (for profiling)")
     ap.add_argument("--workload", default="cfg2", choices=sorted(CONFIGS) + sorted(DIAG), help="headline workload")
     ap.add_argument("--cpu-slices", type=int, default=16)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch one plain elementwise kernel reading and writing 256 MiB each, so that a "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled against a known transfer")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no multi-GPU path exists); use --gpus 1", file=sys.stderr)
@@ -193,6 +212,13 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
+
+    if args.copy_calibration:
+        src = torch.zeros(64 * 1024 * 1024, dtype=torch.float32, device="cuda")  # 256 MiB
+        dst = torch.empty_like(src)
+        torch.add(src, 1.0, out=dst)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     name = args.workload
     c = CONFIGS[name] if name in CONFIGS else DIAG[name]
@@ -208,7 +234,7 @@ def main():
         value, unit = fl / (host_ms * 1e-3) / 1e12, "TFLOP/s"
         roof = {"bound": "mfma", "achieved": fl / (ev_ms * 1e-3) / 1e12, "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = None
+    roof["traffic"] = measured_traffic(name)
     roof["kernel_ms"] = ev_ms
 
     result = {
@@ -244,7 +270,8 @@ def main():
         result["other_workloads"] = others
         if "cfg5" in others:
             result["roofline_decode"] = {"bound": "hbm", "achieved": others["cfg5"]["GB/s"], "peak": PEAK_HBM_GBPS,
-                                         "unit": "GB/s", "frac": others["cfg5"]["frac_hbm_peak"], "traffic": None}
+                                         "unit": "GB/s", "frac": others["cfg5"]["frac_hbm_peak"],
+                                         "traffic": measured_traffic("cfg5")}
     print(json.dumps(result))
 
 
