@@ -1,9 +1,18 @@
-// Instances of the tiled forward kernel for the head-dim bucket d <= 128.
-#include "fwd_kernel.h"
+// Instances of the tiled forward kernels for the head-dim bucket d <= 128.
+#include <cstdlib>
+
+#include "fwd_pp_kernel.h"
 namespace fa {
 int launch_fwd_d128(const FwdArgs& a, int variant, int nb, hipStream_t st)
 {
     (void)nb;
+    // d == 128, more than one 128-row block of queries and no narrow window: the 8-wave ping-pong kernel (measured
+    // 3-12 % faster than the 4-wave kernel there; slower for d = 64 and for windows much smaller than its 256-row
+    // block, which make it compute mostly masked tiles).  FLASH_ATTN_NO_PINGPONG=1 forces the 4-wave kernel (A/B runs).
+    static const bool no_pp = std::getenv("FLASH_ATTN_NO_PINGPONG") != nullptr;
+    const bool narrow_window = (a.wl >= 0 && a.wl < 512) || (a.wr >= 0 && a.wr < 512 && !a.causal);
+    if ((variant & kVarVec) && a.d == 128 && a.Nq > 128 && !narrow_window && !no_pp)
+        return launch_fwd_pp_bucket<128>(a, variant, st);
     return launch_fwd_bucket<128, 1>(a, variant, st);
 }
 }  // namespace fa

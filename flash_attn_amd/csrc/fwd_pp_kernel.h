@@ -1,0 +1,549 @@
+// Ping-pong variant of the tiled forward kernel for head dims 64 and 128 that fill their bucket (d == D).
+//
+// Same math as fwd_kernel.h (S^T = K Q^T and O^T += V^T P^T on MFMA 32x32x16, Q in registers, online softmax per
+// lane, 64-key tiles).  What changes is the schedule and the way tiles reach LDS:
+//
+//  * One work-group = 8 waves = 256 query rows and fills a CU: every SIMD hosts two of its waves (w and w+4).
+//  * Each wave alternates between a VALU phase, softmax(S(t)) -> P(t), and an MFMA phase, O += P(t) V(t) followed by
+//    S(t+1) = K(t+1) Q^T.  Waves 0-3 and waves 4-7 run half an iteration apart: the second group passes one extra
+//    barrier before the loop, and every phase ends in a work-group barrier.  So on every SIMD one wave is in its MFMA
+//    phase while the other is in its VALU phase.  (Two independent 4-wave groups per CU do not interleave this way
+//    by themselves: measured MFMA / VALU co-execution was 11 % of the time.)
+//  * Tiles go from global memory straight into LDS (global_load_lds_dwordx4: 64 lanes write one contiguous KiB, each
+//    lane fetching from its own global address), in a fragment-major layout: the KiB written by one load is exactly
+//    what the 64 lanes of one ds_read_b128 (K fragment) or of two ds_read_b64_tr_b16 (V fragment halves) read back
+//    as base + lane * 16 (resp. * 8).  No staging registers, no ds_write, no padding, conflict-free by construction,
+//    and every LDS read address is one base register plus an immediate.
+//  * Four LDS stages per tensor: K(t+3) and V(t+2) are requested at the start of the VALU phase of iteration t and
+//    waited for (vmcnt) at the end of the MFMA phase of the same iteration; with the half-iteration offset their
+//    slots (K(t-1), V(t-2)) were last read two barriers earlier, and the first reader comes two barriers later.
+//  * Barriers wait for LDS traffic only; the first V fragment reads of a phase are issued before its barrier.
+#pragma once
+#include "fwd_kernel.h"
+
+namespace fa {
+
+template <int D>
+struct PPCfg {
+    static constexpr int kWaves = 8;
+    static constexpr int BR = 32 * kWaves;    // query rows per work-group
+    static constexpr int BC = 64;             // keys per tile
+    static constexpr int KS = D / 16;
+    static constexpr int MB = D / 32;
+    static constexpr int KBUF = BC * D * 2;   // bytes per K stage (fragment-major, unpadded)
+    static constexpr int VBUF = BC * D * 2;
+    static constexpr int NST = 4;             // LDS stages per tensor
+    static constexpr int SMEM = NST * (KBUF + VBUF);
+    static constexpr int NKL = (2 * KS) / 8;  // 1 KiB K blocks loaded per wave per tile
+    static constexpr int NVL = (4 * MB) / 8;  // 1 KiB V blocks loaded per wave per tile
+    static_assert(D == 64 || D == 128, "ping-pong kernel: head dim 64 or 128");
+};
+
+// One KiB from global memory straight into LDS: lane l fetches 16 bytes at base + off (its own offset) and the wave
+// writes them to lds_dst + 16 l.  Issued as inline asm on purpose: the compiler models the builtin form as a FLAT
+// access that may touch LDS, and from then on degrades every LDS wait of the loop to "wait for everything".  The
+// caller waits with s_waitcnt vmcnt(0) before the barrier that publishes the tile.
+__device__ __forceinline__ void dma_kib(const char* base, uint32_t off, FA_LDS char* lds_dst)
+{
+    const uint32_t m0v = (uint32_t)(uintptr_t)lds_dst;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(m0v), "v"(off), "s"(base)
+                 : "memory", "m0");
+}
+
+// LDS-only barrier: global loads in flight are not waited for.
+// The sched_barrier fences keep the compiler from moving ALU work of one phase across the barrier into the other.
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// Barrier between the VALU and the MFMA phase: LDS writes of this wave are done (they were issued before the reads
+// that may still be in flight: LDS operations of a wave complete in order, so waiting until at most `kReads` operations
+// are outstanding covers every write), the first V fragment reads stay in flight across the barrier.
+template <int kReads>
+__device__ __forceinline__ void lds_barrier_keep(void)
+{
+    static_assert(kReads == 8 || kReads == 12 || kReads == 16 || kReads == 4, "");
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (kReads == 16) asm volatile("s_waitcnt lgkmcnt(15)\n\ts_barrier" ::: "memory");
+    else if constexpr (kReads == 12) asm volatile("s_waitcnt lgkmcnt(12)\n\ts_barrier" ::: "memory");
+    else if constexpr (kReads == 8) asm volatile("s_waitcnt lgkmcnt(8)\n\ts_barrier" ::: "memory");
+    else asm volatile("s_waitcnt lgkmcnt(4)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+template <int D, int VAR>
+__global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
+{
+    constexpr bool kAlibi = (VAR & kVarAlibi) != 0, kDropout = (VAR & kVarDropout) != 0;
+    using C = PPCfg<D>;
+    constexpr int BC = C::BC, KS = C::KS, MB = C::MB, NKL = C::NKL, NVL = C::NVL, NST = C::NST;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    FA_LDS char* const Ks = (FA_LDS char*)smem;
+    FA_LDS char* const Vs = Ks + NST * C::KBUF;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = wave_uniform(tid >> 6);
+    const int grp = wave >> 2;  // waves w and w+4 share a SIMD and run half an iteration apart
+    const int l32 = lane & 31;
+    const int g = lane >> 5;
+
+    const int BH = a.B * a.H;
+    const int id = blockIdx.x;
+    const int bh = id % BH;
+    const int rest = id / BH;
+    const int split = rest % a.num_splits;
+    const int m_block = a.Tr - 1 - rest / a.num_splits;
+    const int h = bh % a.H;
+    const int Nq = a.Nq, Nk = a.Nk;
+    constexpr int d = D;
+    const int shift = Nk - Nq;
+    const int q0 = m_block * C::BR;
+
+    // ---- key range of the work-group (same pruning as fwd_kernel)
+    int kmin = 0, kmax = Nk;
+    {
+        const int last_row = (q0 + C::BR - 1 < Nq ? q0 + C::BR - 1 : Nq - 1) + shift;
+        if (a.wl >= 0) kmin = max(0, q0 + shift - a.wl);
+        if (a.causal) kmax = min(kmax, last_row + 1);
+        if (a.wr >= 0) kmax = min(kmax, last_row + a.wr + 1);
+        if (a.num_splits > 1) {
+            const int s0 = split * a.keys_per_split;
+            kmin = max(kmin, s0);
+            kmax = min(kmax, s0 + a.keys_per_split);
+        }
+    }
+    const int tile_begin = kmin / BC;
+    const int ntiles = kmax > kmin ? (kmax + BC - 1) / BC - tile_begin : 0;
+
+    // ---- this lane's query row and its interval of allowed keys
+    // Row block of this wave: SIMD s hosts waves s and s + 4; giving them row blocks s and 7 - s evens out how long
+    // each SIMD stays busy in the causal diagonal, where upper row blocks run out of visible keys first.
+    const int rblk = wave < 4 ? wave : 11 - wave;
+    const int row_i = q0 + rblk * 32 + l32;
+    int lo, hi;
+    float iif;
+    {
+        const int ii = (row_i < Nq ? row_i : Nq - 1) + shift;
+        lo = 0;
+        hi = Nk - 1;
+        if (a.wl >= 0) lo = max(0, ii - a.wl);
+        if (a.causal) hi = min(hi, ii);
+        if (a.wr >= 0) hi = min(hi, ii + a.wr);
+        if (a.num_splits > 1) {
+            lo = max(lo, kmin);
+            hi = min(hi, kmax - 1);
+        }
+        iif = (float)ii;
+    }
+    int lo_max, hi_min;  // wave-uniform: does a tile need the element test at all
+    int lo_min, hi_max;  // wave-uniform: can a tile hold any visible key for this wave
+    {
+        const int first = q0 + rblk * 32, last = first + 31;
+        const int iif_ = (first < Nq ? first : Nq - 1) + shift, iil_ = (last < Nq ? last : Nq - 1) + shift;
+        lo_max = 0;
+        hi_min = Nk - 1;
+        if (a.wl >= 0) lo_max = max(0, iil_ - a.wl);
+        if (a.causal) hi_min = min(hi_min, iif_);
+        if (a.wr >= 0) hi_min = min(hi_min, iif_ + a.wr);
+        if (a.num_splits > 1) {
+            lo_max = max(lo_max, kmin);
+            hi_min = min(hi_min, kmax - 1);
+        }
+        lo_min = 0;
+        hi_max = Nk - 1;
+        if (a.wl >= 0) lo_min = max(0, iif_ - a.wl);
+        if (a.causal) hi_max = min(hi_max, iil_);
+        if (a.wr >= 0) hi_max = min(hi_max, iil_ + a.wr);
+    }
+
+    const half_t* __restrict__ Qbh = a.Q + (size_t)bh * Nq * d;
+    const half_t* __restrict__ Kbh = a.K + (size_t)bh * Nk * d;
+    const half_t* __restrict__ Vbh = a.V + (size_t)bh * Nk * d;
+
+    // ---- Q fragments
+    v8h qf[KS];
+    {
+        const half_t* qrow = Qbh + (size_t)(row_i < Nq ? row_i : Nq - 1) * d;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            union { v4u u; v8h h; } t;
+            t.u = *reinterpret_cast<const v4u*>(qrow + 16 * ks + 8 * g);
+            qf[ks] = t.h;
+        }
+    }
+
+    // ---- direct global -> LDS tile loads.  Block `blk` of a K stage is the fragment (ks = blk / 2, kb = blk % 2):
+    // lane l holds row 32 kb + l % 32, columns 16 ks + 8 (l / 32) .. +7.  KiB `q` of a V stage holds the two transpose-read
+    // blocks tb = 2 q, 2 q + 1, tb = (st * MB + mb) * 2 + h: 16-lane group G of a block holds keys
+    // 16 st + 8 h + 4 (G / 2) + 0..3, columns 32 mb + 16 (G % 2) + 0..15, four keys x 32 bytes in lane order.
+    // Wave w fetches blocks w, w + 8, ...; offsets are bytes from the slice base for the first tile of the group.
+    uint32_t kgo[NKL], vgo[NVL];
+    int vkey[NVL];
+#pragma unroll
+    for (int x = 0; x < NKL; ++x) {
+        const int blk = wave + 8 * x;
+        const int row = 32 * (blk & 1) + l32;
+        kgo[x] = (uint32_t)(((tile_begin * BC + row) * d + 16 * (blk >> 1) + 8 * g) * 2);
+    }
+#pragma unroll
+    for (int x = 0; x < NVL; ++x) {
+        const int tb = 2 * (wave + 8 * x) + g;
+        const int st = tb / (2 * MB), mb = (tb >> 1) % MB, hh = tb & 1;
+        const int j = lane & 31, G = j >> 3, u = j & 7;
+        vkey[x] = 16 * st + 8 * hh + 4 * (G >> 1) + (u >> 1);
+        vgo[x] = (uint32_t)(((tile_begin * BC + vkey[x]) * d + 32 * mb + 16 * (G & 1) + 8 * (u & 1)) * 2);
+    }
+    const char* const Kb = reinterpret_cast<const char*>(Kbh);
+    const char* const Vb = reinterpret_cast<const char*>(Vbh);
+    // tile index t counts from tile_begin; rows past Nk re-read row Nk - 1 (their scores are masked)
+    auto load_k = [&](int t, FA_LDS char* stage) {
+        const uint32_t toff = (uint32_t)t * (uint32_t)(BC * d * 2);
+        const int rows_left = Nk - (tile_begin + t) * BC;  // >= 1
+#pragma unroll
+        for (int x = 0; x < NKL; ++x) {
+            uint32_t o = kgo[x] + toff;
+            if (rows_left < BC) {
+                const int row = 32 * ((wave + 8 * x) & 1) + l32;
+                if (row >= rows_left) o -= (uint32_t)((row - rows_left + 1) * d * 2);
+            }
+            dma_kib(Kb, o, stage + (wave + 8 * x) * 1024);
+        }
+    };
+    auto load_v = [&](int t, FA_LDS char* stage) {
+        const uint32_t toff = (uint32_t)t * (uint32_t)(BC * d * 2);
+        const int rows_left = Nk - (tile_begin + t) * BC;
+#pragma unroll
+        for (int x = 0; x < NVL; ++x) {
+            uint32_t o = vgo[x] + toff;
+            if (rows_left < BC && vkey[x] >= rows_left) o -= (uint32_t)((vkey[x] - rows_left + 1) * d * 2);
+            dma_kib(Vb, o, stage + (wave + 8 * x) * 1024);
+        }
+    };
+
+    // ---- accumulators
+    v16f oacc[MB];
+    float m_ref = -INFINITY, l_run = 0.0f;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[mb][r] = 0.0f;
+
+    const float c2 = a.scale_log2;
+    float slope2 = 0.0f;
+    if constexpr (kAlibi) slope2 = a.alibi ? a.alibi[h] * kLog2e : 0.0f;
+
+    const int k_rd = lane * 16;  // fragment-major: a fragment is read back in lane order
+    const int v_rd = lane * 8;
+
+    v16f s[2];
+    v8h pf[2][2];
+
+    // Fragment registers of the MFMA phase.  The phase is one software-pipelined stream of LDS reads and MFMAs:
+    //   before the barrier : V fragments of key steps 0 and 1 (the tile has been in LDS for a whole iteration)
+    //   PV step st         : MFMAs of step st, reads of step st+2; the last two steps read the first K fragments
+    //   QK step ks         : MFMAs of step ks, reads of step ks+KPD
+    // so that no MFMA waits for a read issued less than ~8 MFMAs earlier.
+    union VF { v4hp p[2]; v8h v; };
+    VF vf[4][MB];
+    constexpr int KPD = KS < 3 ? KS : 3;  // K k-steps in flight
+    v8h kf[KS][2];
+    auto v_read = [&](FA_LDS const char* vbase, int st) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            FA_LDS const char* p0 = vbase + (st * MB + mb) * 1024;
+            vf[st][mb].p[0] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((FA_LDS v4hp*)(p0));
+            vf[st][mb].p[1] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((FA_LDS v4hp*)(p0 + 512));
+        }
+    };
+    auto k_read = [&](FA_LDS const char* kbase, int ks) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) kf[ks][kb] = *reinterpret_cast<FA_LDS const v8h*>(kbase + (2 * ks + kb) * 1024);
+    };
+    // Lane offset inside a fragment block.  It is laundered through an empty asm once per phase: the compiler would
+    // otherwise pre-add it to every per-fragment constant and keep one address register per read, instead of one base
+    // register plus the DS offset field.  (The stage pointers themselves must stay visible: they carry the
+    // no-alias information that separates these reads from the LDS-DMA writes in flight.)
+    auto lane_off = [&](int v) {
+        asm volatile("" : "+v"(v));
+        return v;
+    };
+    auto pv_mfma = [&](int st) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+            oacc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[st][mb].v, pf[st >> 1][st & 1], oacc[mb], 0, 0, 0);
+    };
+    auto qk_mfma = [&](int ks) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks][kb], qf[ks], s[kb], 0, 0, 0);
+    };
+    auto s_clear = [&]() {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[kb][r] = 0.0f;
+    };
+    // stand-alone S^T = K Q^T (prologue only)
+    auto qk = [&](FA_LDS const char* __restrict__ rdk) {
+        FA_LDS const char* kbase = rdk + lane_off(k_rd);
+#pragma unroll
+        for (int ks = 0; ks < KPD; ++ks) k_read(kbase, ks);
+        s_clear();
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (ks + KPD < KS) k_read(kbase, ks + KPD);
+            qk_mfma(ks);
+        }
+    };
+    // MFMA phase body after the barrier: O += P V(t) with the first K(t+1) fragments fetched under its last MFMAs,
+    // then S = K(t+1) Q^T.  One basic block, so that the read / MFMA interleaving below can be pinned.  After the last
+    // tile the K stage holds stale data and the resulting S is never used (one wasted QK per row block).
+    auto mfma_phase = [&](FA_LDS const char* vbase, FA_LDS const char* kbase) {
+        pv_mfma(0);
+        __builtin_amdgcn_sched_barrier(0);  // step 0 first: its fragments were requested first
+        v_read(vbase, 2);
+        pv_mfma(1);
+        v_read(vbase, 3);
+        pv_mfma(2);
+#pragma unroll
+        for (int ks = 0; ks < KPD; ++ks) k_read(kbase, ks);
+        pv_mfma(3);
+        s_clear();
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (ks + KPD < KS) k_read(kbase, ks + KPD);
+            qk_mfma(ks);
+        }
+        // pin the order: [2MB reads][MB MFMA][2MB reads][MB MFMA][2*KPD reads][MB MFMA]{[2 reads][2 MFMA]}...
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * MB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, MB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * MB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, MB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * KPD, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, MB, 0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (ks + KPD < KS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        }
+    };
+
+    // online softmax of the tile whose scores sit in s; leaves P^T packed to fp16 in pf
+    auto softmax = [&](bool need_mask, int kb0) {
+        if constexpr (kAlibi) {
+            const float jb = (float)(kb0 + 4 * g) - iif;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float dist = jb + (float)(32 * kb + 8 * (r >> 2) + (r & 3));
+                    s[kb][r] = s[kb][r] * c2 - slope2 * __builtin_fabsf(dist);
+                }
+        }
+        if (need_mask) {
+            int lo_rel = lo - kb0 - 4 * g, hi_rel = hi - kb0 - 4 * g;
+            asm volatile("; boundary tile: element mask" : "+v"(lo_rel), "+v"(hi_rel));
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int jr = 32 * kb + 8 * (r >> 2) + (r & 3);
+                    if (jr < lo_rel || jr > hi_rel) s[kb][r] = -INFINITY;
+                }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kb][r]);
+        mx = xhalf_max(mx);
+        if constexpr (!kAlibi) mx *= c2;
+        if (__builtin_amdgcn_ballot_w64(mx > m_ref + kLazyTau) != 0ull) {
+            const float m_new = fmaxf(m_ref, mx);
+            float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_ref - m_new);
+            asm volatile("; raise running max" : "+v"(alpha));
+            m_ref = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[mb][r] *= alpha;
+        }
+        const float m_use = (m_ref == -INFINITY) ? 0.0f : m_ref;
+        float rs = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float p;
+                if constexpr (kAlibi) p = fast_exp2(s[kb][r] - m_use);
+                else p = fast_exp2(__builtin_fmaf(s[kb][r], c2, -m_use));
+                rs += p;
+                s[kb][r] = p;
+            }
+        l_run += rs;
+        if constexpr (kDropout) {
+            const uint32_t i_u = (uint32_t)row_i;
+            uint8_t* kout = a.keep_out ? a.keep_out + ((size_t)bh * Nq + row_i) * Nk : nullptr;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int rg = 0; rg < 4; ++rg) {
+                    const int j0 = kb0 + 32 * kb + 8 * rg + 4 * g;
+                    const v4u w = philox4x32_10((uint32_t)(j0 >> 2), i_u, (uint32_t)bh, a.off_lo, a.seed_lo, a.seed_hi);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const bool keep = w[e] >= a.drop_thr;
+                        s[kb][4 * rg + e] = keep ? s[kb][4 * rg + e] * a.drop_rscale : 0.0f;
+                        if (kout && row_i < Nq && j0 + e < Nk) kout[j0 + e] = keep ? 1 : 0;
+                    }
+                }
+        }
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pf[kb][tt][e] = (half_t)s[kb][8 * tt + e];
+    };
+
+    // One iteration.  The four stage pointers are distinct LDS regions; declaring them restrict is what lets the
+    // compiler issue the fragment reads without first waiting (vmcnt) for the LDS-DMA writes into the other stages.
+    auto iteration = [&](FA_LDS const char* __restrict__ rdv, FA_LDS const char* __restrict__ rdk,
+                         FA_LDS char* __restrict__ wrk, FA_LDS char* __restrict__ wrv, int t) {
+        const int kb0 = (tile_begin + t) * BC;
+        // ---------------- VALU phase: request the tiles to come, softmax of tile t
+        if (t + 3 < ntiles) load_k(t + 3, wrk);
+        if (t + 2 < ntiles) load_v(t + 2, wrv);
+        const bool need_mask = (kb0 < lo_max) || (kb0 + BC - 1 > hi_min);
+        softmax(need_mask, kb0);
+        __builtin_amdgcn_sched_barrier(0);
+        FA_LDS const char* vbase = rdv + lane_off(v_rd);
+        FA_LDS const char* kbase = rdk + lane_off(k_rd);
+        v_read(vbase, 0);
+        __builtin_amdgcn_sched_barrier(0);  // keep the request order: step 0 is consumed first
+        v_read(vbase, 1);
+        lds_barrier_keep<4 * MB>();
+        // ---------------- MFMA phase: O += P(t) V(t), then S(t+1) = K(t+1) Q^T
+        __builtin_amdgcn_s_setprio(1);
+        mfma_phase(vbase, kbase);
+        __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of K(t+3), V(t+2) is in LDS
+        lds_barrier();
+    };
+
+    // ---- prologue: K(0..2), V(0..1) requested; everything landed before the first barrier
+    if (ntiles > 0) {
+        load_k(0, Ks);
+        load_v(0, Vs);
+        if (ntiles > 1) {
+            load_k(1, Ks + C::KBUF);
+            load_v(1, Vs + C::VBUF);
+        }
+        if (ntiles > 2) load_k(2, Ks + 2 * C::KBUF);
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));  // Q has landed: no vmcnt waits on qf in the loop
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    lds_barrier();
+    if (ntiles > 0) qk(Ks);
+    if (grp == 1) lds_barrier();  // second wave group runs half an iteration behind
+
+    // Tiles whose keys (and whose successor's keys) are all invisible to this wave contribute nothing: there the wave
+    // only serves its share of the loads and the barriers.  Live tiles form one contiguous range [t_lo, t_hi).
+    auto idle_iteration = [&](int t) {
+        if (t + 3 < ntiles) load_k(t + 3, Ks + ((t + 3) % NST) * C::KBUF);
+        if (t + 2 < ntiles) load_v(t + 2, Vs + ((t + 2) % NST) * C::VBUF);
+        lds_barrier();
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        lds_barrier();
+    };
+    // The full loop starts one tile before the first visible one: that tile is masked entirely (whatever stale scores
+    // the wave holds for it), and its iteration produces the scores of the first visible tile.
+    int t_lo = lo_min / BC - tile_begin - 1;
+    int t_hi = hi_max >= 0 ? hi_max / BC - tile_begin + 1 : 0;  // one past the last tile with a visible key
+    t_lo = t_lo < 0 ? 0 : t_lo;
+    t_hi = t_hi > ntiles ? ntiles : t_hi;
+    if (t_lo > t_hi) t_lo = t_hi;
+    int t = 0;
+    for (; t < t_lo; ++t) idle_iteration(t);
+    for (; t < t_hi; ++t)
+        iteration(Vs + (t % NST) * C::VBUF, Ks + ((t + 1) % NST) * C::KBUF, Ks + ((t + 3) % NST) * C::KBUF,
+                  Vs + ((t + 2) % NST) * C::VBUF, t);
+    for (; t < ntiles; ++t) idle_iteration(t);
+    if (grp == 0) lds_barrier();  // both groups pass the same number of barriers
+
+    // ---------------- epilogue
+    {
+        const float l = xhalf_sum(l_run);
+        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+        const float lse = l > 0.0f ? (m_ref + fast_log2(l)) * kLn2 : -INFINITY;
+        if (row_i < Nq) {
+            if (a.num_splits > 1) {
+                const size_t prow = ((size_t)bh * a.num_splits + split) * Nq + row_i;
+                if (g == 0) a.LSE_partial[prow] = lse;
+                float* op = a.O_partial + prow * d;
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int rg = 0; rg < 4; ++rg) {
+                        const int dc = 32 * mb + 8 * rg + 4 * g;
+                        v4f o = {oacc[mb][4 * rg] * inv, oacc[mb][4 * rg + 1] * inv, oacc[mb][4 * rg + 2] * inv,
+                                 oacc[mb][4 * rg + 3] * inv};
+                        *reinterpret_cast<v4f*>(op + dc) = o;
+                    }
+            } else {
+                if (g == 0) a.LSE[(size_t)bh * Nq + row_i] = lse;
+                half_t* op = a.O + ((size_t)bh * Nq + row_i) * d;
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int rg = 0; rg < 4; ++rg) {
+                        const int dc = 32 * mb + 8 * rg + 4 * g;
+                        v4h o = {(half_t)(oacc[mb][4 * rg] * inv), (half_t)(oacc[mb][4 * rg + 1] * inv),
+                                 (half_t)(oacc[mb][4 * rg + 2] * inv), (half_t)(oacc[mb][4 * rg + 3] * inv)};
+                        *reinterpret_cast<v4h*>(op + dc) = o;
+                    }
+            }
+        }
+    }
+}
+
+template <int D, int VAR>
+inline hipError_t launch_fwd_pp_instance(const FwdArgs& a, hipStream_t st)
+{
+    using C = PPCfg<D>;
+    auto kern = fwd_pp_kernel<D, VAR>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    FwdArgs b = a;
+    b.Tr = (a.Nq + C::BR - 1) / C::BR;
+    const long long groups = (long long)b.Tr * a.B * a.H * a.num_splits;
+    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(512), C::SMEM, st, b);
+    return hipGetLastError();
+}
+
+// d == D, 16-byte rows: {plain, ALiBi, dropout, both}
+template <int D>
+inline int launch_fwd_pp_bucket(const FwdArgs& a, int variant, hipStream_t st)
+{
+    const int feat = variant & (kVarAlibi | kVarDropout);
+    hipError_t e;
+    if (feat == 0) e = launch_fwd_pp_instance<D, 0>(a, st);
+    else if (feat == kVarAlibi) e = launch_fwd_pp_instance<D, kVarAlibi>(a, st);
+    else if (feat == kVarDropout) e = launch_fwd_pp_instance<D, kVarDropout>(a, st);
+    else e = launch_fwd_pp_instance<D, kVarAlibi | kVarDropout>(a, st);
+    return (int)e;
+}
+
+}  // namespace fa
