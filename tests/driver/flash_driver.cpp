@@ -1,0 +1,274 @@
+// Bench + verify driver for libflash_attn_mi355.so: the counterpart of the reference's main() (src/main.cu:38-251)
+// with run-time flags in place of its const locals.  Test infrastructure: it links the CPU oracle as the checker.
+//
+// Same steps as the reference: fill Q/K/V on the host (src/main.cu:91-103: std::default_random_engine(26),
+// U(0,10), drawn in the order Q[i], K[i], V[i]), convert to fp16, copy to the device, pick the split count
+// (src/main.cu:125), one warm-up launch and `--iters` timed launches between two events (src/main.cu:187-213), the
+// CPU forward (src/main.cu:216), then verfiy with a relative bound of 0.06 (src/main.cu:221-224, 254-276).
+// The printed lines ("split_num: ", "kernel time: ... us", the verfiy banner) keep the reference's wording so that
+// logs can be compared side by side.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "flash_attn_mi355.h"
+
+extern "C" {
+// oracle/attention_oracle.c
+int oracle_attention_forward(const float* Q, const float* K, const float* V, int B, int H, int Nq, int Nk, int d,
+                             float scale, int causal, int window_left, int window_right, const float* slopes,
+                             const uint8_t* keep_mask, float p_drop, float* O, float* LSE, int nthreads);
+int oracle_max_threads(void);
+}
+
+namespace {
+
+struct Options {
+    int batch = 1, heads = 8, seq = 1021, head_dim = 31;  // the reference's defaults, src/main.cu:39-42
+    bool causal = false, alibi = false, verify = true;
+    int window = -1;
+    float dropout = 0.0f;
+    int splits = 0;  // 0: library heuristic, > 0: explicit
+    int iters = 1000, warmup = 1;
+    float tol = 0.06f;
+    long long max_print = 20;
+    std::string fill = "reference";
+};
+
+void usage(const char* argv0)
+{
+    std::printf(
+        "usage: %s [options]\n"
+        "  --batch B --heads H --seq N --head-dim d     problem size (default 1 8 1021 31, as src/main.cu:39-42)\n"
+        "  --causal                                     causal mask\n"
+        "  --window W                                   local attention, W keys to either side (reference: 128)\n"
+        "  --alibi                                      per-head slopes -2^(-8(h+1)/H) as in src/main.cu:65-67\n"
+        "  --dropout P                                  dropout probability (disables the check, as the reference does)\n"
+        "  --splits S                                   key splits: 0 = heuristic (default), S > 0 explicit\n"
+        "  --iters K --warmup W                         timed / untimed launches (default 1000 / 1)\n"
+        "  --fill reference|normal                      U(0,10) with engine seed 26 (default) or N(0,1), seed 26\n"
+        "  --tol T                                      relative error bound of the check (default 0.06)\n"
+        "  --max-print M                                print at most M mismatches (default 20, -1: all)\n"
+        "  --no-verify                                  skip the CPU forward and the check\n",
+        argv0);
+}
+
+bool parse(int argc, char** argv, Options* o)
+{
+    for (int i = 1; i < argc; ++i) {
+        const std::string a = argv[i];
+        auto next = [&](const char* what) -> const char* {
+            if (i + 1 >= argc) {
+                std::fprintf(stderr, "%s needs a value\n", what);
+                std::exit(2);
+            }
+            return argv[++i];
+        };
+        if (a == "--batch") o->batch = std::atoi(next("--batch"));
+        else if (a == "--heads") o->heads = std::atoi(next("--heads"));
+        else if (a == "--seq") o->seq = std::atoi(next("--seq"));
+        else if (a == "--head-dim") o->head_dim = std::atoi(next("--head-dim"));
+        else if (a == "--causal") o->causal = true;
+        else if (a == "--window") o->window = std::atoi(next("--window"));
+        else if (a == "--alibi") o->alibi = true;
+        else if (a == "--dropout") o->dropout = (float)std::atof(next("--dropout"));
+        else if (a == "--splits") o->splits = std::atoi(next("--splits"));
+        else if (a == "--iters") o->iters = std::atoi(next("--iters"));
+        else if (a == "--warmup") o->warmup = std::atoi(next("--warmup"));
+        else if (a == "--fill") o->fill = next("--fill");
+        else if (a == "--tol") o->tol = (float)std::atof(next("--tol"));
+        else if (a == "--max-print") o->max_print = std::atoll(next("--max-print"));
+        else if (a == "--no-verify") o->verify = false;
+        else if (a == "--help" || a == "-h") return false;
+        else {
+            std::fprintf(stderr, "unknown option %s\n", a.c_str());
+            return false;
+        }
+    }
+    if (o->batch < 1 || o->heads < 1 || o->seq < 1 || o->head_dim < 1 || o->iters < 1 || o->warmup < 0) return false;
+    if (o->fill != "reference" && o->fill != "normal") return false;
+    return true;
+}
+
+#define HIP_CHECK(call)                                                                              \
+    do {                                                                                             \
+        hipError_t e_ = (call);                                                                      \
+        if (e_ != hipSuccess) {                                                                      \
+            std::fprintf(stderr, "HIP error: %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+            std::exit(1);                                                                            \
+        }                                                                                            \
+    } while (0)
+
+// verfiy of src/main.cu:254-276 with the same predicate and banner; printing is capped by max_print
+long long verfiy(const float* O, const float* O_host, long long n, float range_of_error, long long max_print)
+{
+    long long error = 0;
+    std::printf("===================start verfiy===================\n");
+    for (long long i = 0; i < n; i++) {
+        const float device_out = O_host[i];
+        if ((std::fabs(O_host[i] - O[i])) / O[i] > range_of_error || std::isnan(device_out) || std::isinf(device_out)) {
+            if (max_print < 0 || error < max_print)
+                std::printf("error, postion:%lld, gpuvalue:%f, cpuvalue:%f\n", i, O_host[i], O[i]);
+            error++;
+        }
+    }
+    std::printf("==================finish,error:%lld==================\n", error);
+    return error;
+}
+
+}  // namespace
+
+int main(int argc, char** argv)
+{
+    Options opt;
+    if (!parse(argc, argv, &opt)) {
+        usage(argv[0]);
+        return 2;
+    }
+    const int B = opt.batch, H = opt.heads, N = opt.seq, d = opt.head_dim;
+    const size_t n = (size_t)B * H * N * d;
+
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) {
+        std::fprintf(stderr, "%s\n", flash_strerror(FLASH_ENODEVICE));
+        return 1;
+    }
+
+    // ---- host data (fill order of src/main.cu:91-103)
+    std::vector<float> Q(n), K(n), V(n), O(n, 0.0f), O_host(n);
+    std::vector<_Float16> Qh(n), Kh(n), Vh(n), Oh(n);
+    {
+        std::default_random_engine generator(26);
+        std::uniform_real_distribution<float> uniform(0.0f, 10.0f);
+        std::normal_distribution<float> normal(0.0f, 1.0f);
+        const bool ref = opt.fill == "reference";
+        for (size_t i = 0; i < n; i++) {
+            Q[i] = ref ? uniform(generator) : normal(generator);
+            K[i] = ref ? uniform(generator) : normal(generator);
+            V[i] = ref ? uniform(generator) : normal(generator);
+            Qh[i] = (_Float16)Q[i];
+            Kh[i] = (_Float16)K[i];
+            Vh[i] = (_Float16)V[i];
+        }
+    }
+    std::vector<float> slopes;
+    float* slopes_dev = nullptr;
+    if (opt.alibi) {
+        slopes.resize(H);
+        for (int i = 0; i < H; i++) slopes[i] = (float)-std::pow(2, -8.0 / H * (i + 1));  // src/main.cu:65-67
+        HIP_CHECK(hipMalloc((void**)&slopes_dev, H * sizeof(float)));
+        HIP_CHECK(hipMemcpy(slopes_dev, slopes.data(), H * sizeof(float), hipMemcpyHostToDevice));
+    }
+
+    void *Qd, *Kd, *Vd, *Od;
+    float* LSEd;
+    HIP_CHECK(hipMalloc(&Qd, n * 2));
+    HIP_CHECK(hipMalloc(&Kd, n * 2));
+    HIP_CHECK(hipMalloc(&Vd, n * 2));
+    HIP_CHECK(hipMalloc(&Od, n * 2));
+    HIP_CHECK(hipMalloc((void**)&LSEd, (size_t)B * H * N * sizeof(float)));
+    HIP_CHECK(hipMemcpy(Qd, Qh.data(), n * 2, hipMemcpyHostToDevice));
+    HIP_CHECK(hipMemcpy(Kd, Kh.data(), n * 2, hipMemcpyHostToDevice));
+    HIP_CHECK(hipMemcpy(Vd, Vh.data(), n * 2, hipMemcpyHostToDevice));
+
+    flash_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.Q = Qd;
+    p.K = Kd;
+    p.V = Vd;
+    p.O = Od;
+    p.LSE = LSEd;
+    p.B = B;
+    p.H = H;
+    p.Nq = p.Nk = N;
+    p.d = d;
+    p.softmax_scale = (float)(1.0 / std::sqrt((double)d));
+    p.is_causal = opt.causal ? 1 : 0;
+    p.window_left = p.window_right = opt.window;
+    p.alibi_slopes = slopes_dev;
+    p.dropout_p = opt.dropout;
+    p.seed = 48;  // src/main.cu:134
+    p.offset = 0;
+    p.num_splits = opt.splits;
+
+    const int split_num = flash_splitkv_resolve_splits(&p);
+    if (split_num < 1) {
+        std::fprintf(stderr, "%s\n", flash_strerror(split_num));
+        return 1;
+    }
+    std::printf("split_num: %d\n", split_num);
+    p.num_splits = split_num;
+    size_t ob = 0, lb = 0;
+    int rc = flash_splitkv_workspace_bytes(&p, &ob, &lb);
+    if (rc != FLASH_OK) {
+        std::fprintf(stderr, "%s\n", flash_strerror(rc));
+        return 1;
+    }
+    if (ob) {
+        HIP_CHECK(hipMalloc((void**)&p.O_partial, ob));
+        HIP_CHECK(hipMalloc((void**)&p.LSE_partial, lb));
+    }
+
+    auto launch = [&]() {
+        const int e = flash_forward_splitkv(&p, nullptr);
+        if (e != FLASH_OK) {
+            std::fprintf(stderr, "%s (%s)\n", flash_strerror(e), flash_last_hip_error());
+            std::exit(1);
+        }
+    };
+    for (int i = 0; i < opt.warmup; i++) launch();
+
+    hipEvent_t start, stop;
+    HIP_CHECK(hipEventCreate(&start));
+    HIP_CHECK(hipEventCreate(&stop));
+    HIP_CHECK(hipEventRecord(start, 0));
+    for (int i = 0; i < opt.iters; i++) launch();
+    HIP_CHECK(hipGetLastError());
+    HIP_CHECK(hipEventRecord(stop, 0));
+    HIP_CHECK(hipEventSynchronize(stop));
+    float time_elapsed = 0.0f;
+    HIP_CHECK(hipEventElapsedTime(&time_elapsed, start, stop));
+
+    HIP_CHECK(hipMemcpy(Oh.data(), Od, n * 2, hipMemcpyDeviceToHost));
+    for (size_t i = 0; i < n; i++) O_host[i] = (float)Oh[i];
+    // the reference prints the total of its 1000 launches in ms, which is the time of one launch in us
+    std::printf("kernel time: %f us\n", time_elapsed * 1000.0f / (float)opt.iters);
+
+    long long errors = 0;
+    if (opt.verify && opt.dropout == 0.0f) {
+        // the CPU forward sees what the kernel sees: the fp16-rounded inputs
+        for (size_t i = 0; i < n; i++) {
+            Q[i] = (float)Qh[i];
+            K[i] = (float)Kh[i];
+            V[i] = (float)Vh[i];
+        }
+        rc = oracle_attention_forward(Q.data(), K.data(), V.data(), B, H, N, N, d, p.softmax_scale, p.is_causal, opt.window,
+                                      opt.window, opt.alibi ? slopes.data() : nullptr, nullptr, 0.0f, O.data(), nullptr,
+                                      oracle_max_threads());
+        if (rc != 0) {
+            std::fprintf(stderr, "CPU forward failed (%d)\n", rc);
+            return 1;
+        }
+        std::printf("Verify the result of kernel function\n");
+        errors = verfiy(O.data(), O_host.data(), (long long)n, opt.tol, opt.max_print);
+    }
+
+    HIP_CHECK(hipEventDestroy(start));
+    HIP_CHECK(hipEventDestroy(stop));
+    HIP_CHECK(hipFree(Qd));
+    HIP_CHECK(hipFree(Kd));
+    HIP_CHECK(hipFree(Vd));
+    HIP_CHECK(hipFree(Od));
+    HIP_CHECK(hipFree(LSEd));
+    if (p.O_partial) HIP_CHECK(hipFree(p.O_partial));
+    if (p.LSE_partial) HIP_CHECK(hipFree(p.LSE_partial));
+    if (slopes_dev) HIP_CHECK(hipFree(slopes_dev));
+    return errors == 0 ? 0 : 3;
+}

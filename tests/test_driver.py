@@ -1,0 +1,66 @@
+"""The bench + verify driver (tests/driver/flash_driver, counterpart of the reference's main(), src/main.cu:38-251).
+
+CPU: the binary exists, links against the library and the oracle, and rejects bad flags.
+GPU: reference-compatible runs (U(0,10) fill with engine seed 26, verfiy with the 0.06 relative bound of
+src/main.cu:224) must end with "finish,error:0" -- the line the reference prints for a correct kernel.
+"""
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DRIVER = os.path.join(ROOT, "tests", "driver", "flash_driver")
+
+
+def _run(*args, timeout=120):
+    return subprocess.run([DRIVER, *args], capture_output=True, text=True, timeout=timeout)
+
+
+def test_driver_is_built_and_prints_usage():
+    assert os.path.exists(DRIVER), "run `make -C tests/driver` (or __graft_entry__.build())"
+    r = _run("--help")
+    assert r.returncode == 2
+    for flag in ("--batch", "--causal", "--window", "--alibi", "--dropout", "--splits", "--iters", "--fill", "--tol"):
+        assert flag in r.stdout
+    assert _run("--no-such-flag").returncode == 2
+    assert _run("--seq", "0").returncode == 2
+
+
+def _check(out):
+    assert re.search(r"^split_num: \d+$", out, re.M), out
+    assert re.search(r"^kernel time: [0-9.]+ us$", out, re.M), out
+    assert "Verify the result of kernel function" in out
+    assert "===================start verfiy===================" in out
+    m = re.search(r"==================finish,error:(\d+)==================", out)
+    assert m, out
+    return int(m.group(1))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize(
+    "args",
+    [
+        (),  # the reference's own configuration: B1 H8 N1021 d31, split by the heuristic, ragged N and d
+        ("--causal",),
+        ("--window", "128"),
+        ("--alibi",),
+        ("--causal", "--splits", "1"),
+        ("--batch", "2", "--heads", "4", "--seq", "640", "--head-dim", "128", "--causal"),
+        ("--batch", "2", "--heads", "4", "--seq", "512", "--head-dim", "64", "--fill", "normal", "--tol", "1e9"),
+    ],
+    ids=["reference_default", "causal", "window128", "alibi", "causal_nosplit", "d128_causal", "normal_fill"],
+)
+def test_driver_reference_compatible_runs(args):
+    r = _run("--iters", "5", *args)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert _check(r.stdout) == 0
+
+
+@pytest.mark.gpu
+def test_driver_dropout_skips_the_check():
+    # src/main.cu:222: with dropout the CPU result cannot match, so the reference does not verify
+    r = _run("--iters", "3", "--dropout", "0.1", "--seq", "256", "--head-dim", "64")
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "kernel time" in r.stdout and "start verfiy" not in r.stdout
