@@ -14,6 +14,7 @@ import argparse
 import json
 import math
 import os
+import subprocess
 import sys
 import time
 
@@ -157,6 +158,19 @@ def time_steps(step, steps, warmup):
     return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
 
 
+def mfma_sustained():
+    """Sustained 32x32x16 fp16 MFMA rate of this GPU for zero / constant / random operands, measured by the stand-alone
+    probe tests/driver/mfma_rate (a child process; a fraction of a second).  None when the probe is not built."""
+    exe = os.path.join(ROOT, "tests", "driver", "mfma_rate")
+    if not os.path.exists(exe):
+        return None
+    try:
+        out = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+        return json.loads(out.stdout.strip().splitlines()[-1]) if out.returncode == 0 else None
+    except (OSError, ValueError, IndexError, subprocess.TimeoutExpired):
+        return None
+
+
 def cpu_baseline(c, q, k, v, budget_slices):
     """The reference's own attention_forward_cpu (oracle/_ref, compiled from the reference checkout) on a bounded
     sample of (b,h) slices, one core as in the reference; falls back to the restatement when _ref is absent."""
@@ -236,6 +250,13 @@ def main():
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = measured_traffic(name)
     roof["kernel_ms"] = ev_ms
+    if roof["bound"] == "mfma" and not args.only_main:
+        # `peak` is the published figure; what the MFMA pipe of this GPU sustains on changing random operands (with no
+        # other work at all) is measured beside it, since the power management makes it data dependent
+        sus = mfma_sustained()
+        if sus:
+            roof["mfma_sustained"] = sus
+            roof["frac_of_sustained_random"] = roof["achieved"] / sus["random"]
 
     result = {
         "metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

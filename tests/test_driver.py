@@ -28,6 +28,22 @@ def test_driver_is_built_and_prints_usage():
     assert _run("--seq", "0").returncode == 2
 
 
+def test_mfma_rate_probe_is_built():
+    assert os.path.exists(os.path.join(ROOT, "tests", "driver", "mfma_rate")), "run `make -C tests/driver`"
+
+
+@pytest.mark.gpu
+def test_mfma_rate_probe_reports_three_rates():
+    import json
+
+    r = subprocess.run([os.path.join(ROOT, "tests", "driver", "mfma_rate")], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    rates = json.loads(r.stdout.strip().splitlines()[-1])
+    assert rates["unit"] == "TFLOP/s"
+    # nothing can run above the published dense fp16 peak; random operands never run faster than zeros (+5 % noise)
+    assert 100.0 < rates["random"] <= rates["zeros"] * 1.05 <= 2500.0 * 1.05
+
+
 def _check(out):
     assert re.search(r"^split_num: \d+$", out, re.M), out
     assert re.search(r"^kernel time: [0-9.]+ us$", out, re.M), out
