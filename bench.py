@@ -54,6 +54,8 @@ DIAG = {
     "diag_noncausal": dict(B=4, H=16, Nq=2048, Nk=2048, d=128, causal=False, window=(-1, -1), alibi=False, p=0.0, splits=0),
     "diag_d64": dict(B=4, H=16, Nq=2048, Nk=2048, d=64, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=0),
     "diag_long": dict(B=1, H=16, Nq=8192, Nk=8192, d=128, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=0),
+    "diag_gqa_decode": dict(B=16, H=32, Hk=4, Nq=1, Nk=16384, d=128, causal=False, window=(-1, -1), alibi=False, p=0.0,
+                            splits=16),
 }
 DESCR = {
     "cfg1": "plain fwd B=1 H=2 Nq=Nk=128 d=64",
@@ -64,6 +66,7 @@ DESCR = {
     "diag_noncausal": "non-causal fwd B=4 H=16 Nq=Nk=2048 d=128 (diagnostic)",
     "diag_d64": "causal fwd B=4 H=16 Nq=Nk=2048 d=64 (diagnostic)",
     "diag_long": "causal fwd B=1 H=16 Nq=Nk=8192 d=128 (diagnostic)",
+    "diag_gqa_decode": "split-KV decode, 8 query heads per K/V head, B=16 H=32 H_kv=4 Nq=1 Nk=16384 d=128 (diagnostic)",
 }
 
 
@@ -89,7 +92,7 @@ def flops_of(c):
 
 
 def decode_bytes(c):
-    kv = 2 * c["B"] * c["H"] * c["Nk"] * c["d"] * 2
+    kv = 2 * c["B"] * c.get("Hk", c["H"]) * c["Nk"] * c["d"] * 2
     q = c["B"] * c["H"] * c["Nq"] * c["d"] * 2
     o = c["B"] * c["H"] * c["Nq"] * c["d"] * 2
     lse = c["B"] * c["H"] * c["Nq"] * 4
@@ -101,9 +104,9 @@ def make_inputs(c, seed=0):
 
     g = torch.Generator(device="cuda")
     out = []
-    for n, s in ((c["Nq"], 1), (c["Nk"], 2), (c["Nk"], 3)):
+    for n, s, heads in ((c["Nq"], 1, c["H"]), (c["Nk"], 2, c.get("Hk", c["H"])), (c["Nk"], 3, c.get("Hk", c["H"]))):
         g.manual_seed(3 * seed + s)
-        out.append(torch.randn((c["B"], c["H"], n, c["d"]), generator=g, device="cuda", dtype=torch.float32).half())
+        out.append(torch.randn((c["B"], heads, n, c["d"]), generator=g, device="cuda", dtype=torch.float32).half())
     return out
 
 
@@ -239,7 +242,7 @@ def main():
     q, k, v = make_inputs(c)
     step, _ = make_step(fa, c, q, k, v)
     host_ms, ev_ms = time_steps(step, args.steps, args.warmup)
-    if name == "cfg5":
+    if c["Nq"] == 1:
         by = decode_bytes(c)
         value, unit = by / (host_ms * 1e-3) / 1e9, "GB/s"
         roof = {"bound": "hbm", "achieved": by / (ev_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBPS, "unit": "GB/s"}

@@ -37,6 +37,7 @@ class FlashParams(C.Structure):
         ("seed", C.c_uint64), ("offset", C.c_uint64),
         ("num_splits", C.c_int),
         ("keep_mask_out", C.c_void_p),
+        ("H_kv", C.c_int),
     ]
 
 
@@ -104,8 +105,9 @@ def _check_qkv(q, k, v):
         if t.dtype != torch.float16 or not t.is_cuda or not t.is_contiguous():
             raise ValueError("Q, K, V must be contiguous fp16 device tensors")
     B, H, Nq, d = q.shape
-    if k.shape[0] != B or k.shape[1] != H or k.shape[3] != d or v.shape != k.shape:
-        raise ValueError("K, V must be [B,H,Nk,d] matching Q")
+    Hk = k.shape[1]
+    if k.shape[0] != B or Hk < 1 or H % Hk != 0 or k.shape[3] != d or v.shape != k.shape:
+        raise ValueError("K, V must be [B,H_kv,Nk,d] matching Q, with H a multiple of H_kv")
     return B, H, Nq, k.shape[2], d
 
 
@@ -124,6 +126,7 @@ def make_params(q, k, v, o, lse, softmax_scale=None, causal=False, window=(-1, -
     p.seed, p.offset = int(seed), int(offset)
     p.num_splits = int(num_splits)
     p.keep_mask_out = _ptr(keep_mask_out)
+    p.H_kv = int(k.shape[1])
     return p
 
 

@@ -35,6 +35,7 @@ struct FwdArgs {
     const float* alibi;  // [H] or nullptr
     uint8_t* keep_out;   // [B,H,Nq,Nk] or nullptr
     int B, H, Nq, Nk, d;
+    int Hk, kv_group;    // K/V heads and query heads per K/V head (H = Hk * kv_group)
     int causal, wl, wr;  // wl / wr < 0: unbounded
     float scale_log2;    // softmax_scale * log2(e)
     uint32_t drop_thr;   // keep iff philox word >= drop_thr
@@ -43,6 +44,9 @@ struct FwdArgs {
     int num_splits;      // 1: write O/LSE; > 1: write the partial workspace
     int keys_per_split;  // multiple of 128
     int Tr;              // number of query row blocks
+
+    // index of the K/V slice [Nk,d] read by query slice bh = b * H + h
+    __device__ __forceinline__ int kv_slice(int bh) const { return (bh / H) * Hk + (bh % H) / kv_group; }
 };
 
 __device__ __forceinline__ int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }

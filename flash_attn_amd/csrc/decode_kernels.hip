@@ -2,7 +2,8 @@
 //
 // decode_split_kernel replaces forward_kernel_splitkv (src/flash_forward_splitkv.h:14-344) for Nq == 1, where the
 // reference's 128-row MMA tile would waste 127 of 128 rows: the work is a pure stream over K and V, bound by HBM.
-//   * one work-group per (head slice, split); its 4 waves take 128-byte-per-lane blocks of the split's keys in turn
+//   * one work-group per (head slice, split) -- per (G query heads of one K/V head, split) under grouped-query
+//     attention, so that K and V are streamed once per K/V head; its 4 waves take blocks of the split's keys in turn
 //   * a key row is spread over LPK lanes (16 bytes each), so one wave instruction reads 1 KiB of consecutive bytes
 //   * q.k: v_dot2_f32_f16 per lane, then a DPP butterfly over the LPK lanes of the key (no LDS, no shuffles)
 //   * online softmax per key group; p * V accumulated in fp32 per lane (8 head-dim columns per lane)
@@ -31,14 +32,16 @@ __device__ __forceinline__ float group_sum(float v)
     return v;
 }
 
-template <int LPK, bool kAlibi>
+// G = query heads served by one work-group: the G consecutive heads share one K/V head (grouped-query attention), so
+// the K/V stream is read once for all of them.  G == 1 is the plain one-K/V-head-per-query-head case.
+template <int LPK, bool kAlibi, int G>
 __global__ void __launch_bounds__(256) decode_split_kernel(const FwdArgs a)
 {
-    constexpr int KPI = 64 / LPK;  // keys per wave instruction
-    constexpr int U = 8;           // load instructions in flight per tensor
-    constexpr int KB = U * KPI;    // keys per wave block
-    constexpr int NG = 4 * KPI;    // key groups per work-group
-    constexpr int DB = LPK * 8;    // head-dim bucket
+    constexpr int KPI = 64 / LPK;      // keys per wave instruction
+    constexpr int U = G > 2 ? 4 : 8;   // load instructions in flight per tensor
+    constexpr int KB = U * KPI;        // keys per wave block
+    constexpr int NG = 4 * KPI;        // key groups per work-group
+    constexpr int DB = LPK * 8;        // head-dim bucket
     __shared__ float s_acc[NG][DB];
     __shared__ float s_m[NG], s_l[NG];
 
@@ -47,19 +50,21 @@ __global__ void __launch_bounds__(256) decode_split_kernel(const FwdArgs a)
     const int wave = tid >> 6;
     const int c = lane % LPK;
     const int kg = lane / LPK;
-    const int BH = a.B * a.H;
-    const int bh = blockIdx.x % BH;
-    const int split = blockIdx.x / BH;
-    const int h = bh % a.H;
+    const int BHG = a.B * a.H / G;
+    const int bh0 = (blockIdx.x % BHG) * G;  // first of the G query slices of this work-group
+    const int split = blockIdx.x / BHG;
     const int d = a.d, Nk = a.Nk;
     const int col = 8 * c;
     const bool cvalid = col < d;
     const int colc = cvalid ? col : d - 8;
 
     union U8 { v4u u; v8h h; v2h p[4]; };
-    U8 qv;
-    qv.u = *reinterpret_cast<const v4u*>(a.Q + (size_t)bh * d + colc);
-    if (!cvalid) qv.u = v4u{0u, 0u, 0u, 0u};
+    U8 qv[G];
+#pragma unroll
+    for (int gq = 0; gq < G; ++gq) {
+        qv[gq].u = *reinterpret_cast<const v4u*>(a.Q + (size_t)(bh0 + gq) * d + colc);
+        if (!cvalid) qv[gq].u = v4u{0u, 0u, 0u, 0u};
+    }
 
     // the single query row sits at position ii = Nk - 1 (row index i + Nk - Nq): causal / right window never cut
     const int ii = Nk - 1;
@@ -69,16 +74,26 @@ __global__ void __launch_bounds__(256) decode_split_kernel(const FwdArgs a)
         kstart = max(kstart, split * a.keys_per_split);
         kend = min(kend, (split + 1) * a.keys_per_split);
     }
-    const half_t* __restrict__ Kbh = a.K + (size_t)bh * Nk * d + colc;
-    const half_t* __restrict__ Vbh = a.V + (size_t)bh * Nk * d + colc;
+    const int kvs = a.kv_slice(bh0);
+    const half_t* __restrict__ Kbh = a.K + (size_t)kvs * Nk * d + colc;
+    const half_t* __restrict__ Vbh = a.V + (size_t)kvs * Nk * d + colc;
     const float c2 = a.scale_log2;
-    float slope2 = 0.0f;
-    if constexpr (kAlibi) slope2 = a.alibi ? a.alibi[h] * kLog2e : 0.0f;
-
-    float m = -INFINITY, l = 0.0f;
-    float acc[8];
+    float slope2[G];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+    for (int gq = 0; gq < G; ++gq) {
+        slope2[gq] = 0.0f;
+        if constexpr (kAlibi) slope2[gq] = a.alibi ? a.alibi[(bh0 + gq) % a.H] * kLog2e : 0.0f;
+    }
+
+    float m[G], l[G];
+    float acc[G][8];
+#pragma unroll
+    for (int gq = 0; gq < G; ++gq) {
+        m[gq] = -INFINITY;
+        l[gq] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[gq][e] = 0.0f;
+    }
 
     for (int kb = kstart + wave * KB; kb < kend; kb += 4 * KB) {
         U8 kr[U], vr[U];
@@ -94,68 +109,76 @@ __global__ void __launch_bounds__(256) decode_split_kernel(const FwdArgs a)
             const size_t off = (size_t)(j < kend ? j : kend - 1) * d;
             vr[i].u = *reinterpret_cast<const v4u*>(Vbh + off);
         }
-        float t[U];
-        float mb = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < U; ++i) {
-            float s = 0.0f;
+        for (int gq = 0; gq < G; ++gq) {
+            float t[U];
+            float mb = -INFINITY;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) s = __builtin_amdgcn_fdot2(qv.p[e], kr[i].p[e], s, false);
-            s = group_sum<LPK>(s);
-            const int j = kb + i * KPI + kg;
-            float tv = s * c2;
-            if constexpr (kAlibi) tv -= slope2 * (float)(ii - j);
-            if (j >= kend) tv = -INFINITY;
-            t[i] = tv;
-            mb = fmaxf(mb, tv);
+            for (int i = 0; i < U; ++i) {
+                float s = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) s = __builtin_amdgcn_fdot2(qv[gq].p[e], kr[i].p[e], s, false);
+                s = group_sum<LPK>(s);
+                const int j = kb + i * KPI + kg;
+                float tv = s * c2;
+                if constexpr (kAlibi) tv -= slope2[gq] * (float)(ii - j);
+                if (j >= kend) tv = -INFINITY;
+                t[i] = tv;
+                mb = fmaxf(mb, tv);
+            }
+            const float m_new = fmaxf(m[gq], mb);
+            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+            const float alpha = fast_exp2(m[gq] - m_use);
+            m[gq] = m_new;
+            float rs = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[gq][e] *= alpha;
+#pragma unroll
+            for (int i = 0; i < U; ++i) {
+                const float p = fast_exp2(t[i] - m_use);
+                rs += p;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[gq][e] = __builtin_fmaf(p, (float)vr[i].h[e], acc[gq][e]);
+            }
+            l[gq] = l[gq] * alpha + rs;
         }
-        const float m_new = fmaxf(m, mb);
-        const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-        const float alpha = fast_exp2(m - m_use);
-        m = m_new;
-        float rs = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] *= alpha;
-#pragma unroll
-        for (int i = 0; i < U; ++i) {
-            const float p = fast_exp2(t[i] - m_use);
-            rs += p;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(p, (float)vr[i].h[e], acc[e]);
-        }
-        l = l * alpha + rs;
     }
 
-    // ---- merge the NG key groups of the work-group
+    // ---- merge the NG key groups of the work-group, one query head after the other through the same LDS buffer
     const int grp = wave * KPI + kg;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) s_acc[grp][col + e] = acc[e];
-    if (c == 0) {
-        s_m[grp] = m;
-        s_l[grp] = l;
-    }
-    __syncthreads();
-    if (tid < DB) {
-        float M = -INFINITY;
+    for (int gq = 0; gq < G; ++gq) {
+        if (gq > 0) __syncthreads();
 #pragma unroll
-        for (int gI = 0; gI < NG; ++gI) M = fmaxf(M, s_m[gI]);
-        const float Mu = (M == -INFINITY) ? 0.0f : M;
-        float L = 0.0f, o = 0.0f;
-#pragma unroll
-        for (int gI = 0; gI < NG; ++gI) {
-            const float w = fast_exp2(s_m[gI] - Mu);
-            L += w * s_l[gI];
-            o += w * s_acc[gI][tid];
+        for (int e = 0; e < 8; ++e) s_acc[grp][col + e] = acc[gq][e];
+        if (c == 0) {
+            s_m[grp] = m[gq];
+            s_l[grp] = l[gq];
         }
-        const float inv = L > 0.0f ? 1.0f / L : 0.0f;
-        const float lse = L > 0.0f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
-        if (a.num_splits > 1) {
-            const size_t prow = (size_t)bh * a.num_splits + split;  // Nq == 1
-            if (tid < d) a.O_partial[prow * d + tid] = o * inv;
-            if (tid == 0) a.LSE_partial[prow] = lse;
-        } else {
-            if (tid < d) a.O[(size_t)bh * d + tid] = (half_t)(o * inv);
-            if (tid == 0) a.LSE[bh] = lse;
+        __syncthreads();
+        if (tid < DB) {
+            const int bh = bh0 + gq;
+            float M = -INFINITY;
+#pragma unroll
+            for (int gI = 0; gI < NG; ++gI) M = fmaxf(M, s_m[gI]);
+            const float Mu = (M == -INFINITY) ? 0.0f : M;
+            float L = 0.0f, o = 0.0f;
+#pragma unroll
+            for (int gI = 0; gI < NG; ++gI) {
+                const float w = fast_exp2(s_m[gI] - Mu);
+                L += w * s_l[gI];
+                o += w * s_acc[gI][tid];
+            }
+            const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+            const float lse = L > 0.0f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
+            if (a.num_splits > 1) {
+                const size_t prow = (size_t)bh * a.num_splits + split;  // Nq == 1
+                if (tid < d) a.O_partial[prow * d + tid] = o * inv;
+                if (tid == 0) a.LSE_partial[prow] = lse;
+            } else {
+                if (tid < d) a.O[(size_t)bh * d + tid] = (half_t)(o * inv);
+                if (tid == 0) a.LSE[bh] = lse;
+            }
         }
     }
 }
@@ -217,20 +240,29 @@ __global__ void __launch_bounds__(256) keep_mask_kernel(uint8_t* __restrict__ ma
     }
 }
 
+template <int LPK, int G>
+static void launch_decode_instance(const FwdArgs& a, hipStream_t st)
+{
+    const unsigned groups = (unsigned)((long long)a.B * a.H / G * a.num_splits);
+    if (a.alibi != nullptr) hipLaunchKernelGGL((decode_split_kernel<LPK, true, G>), dim3(groups), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((decode_split_kernel<LPK, false, G>), dim3(groups), dim3(256), 0, st, a);
+}
+
+template <int LPK>
+static void launch_decode_bucket(const FwdArgs& a, hipStream_t st)
+{
+    // as many of the query heads of a K/V head per work-group as divide the group (up to 8)
+    if (a.kv_group % 8 == 0) launch_decode_instance<LPK, 8>(a, st);
+    else if (a.kv_group % 4 == 0) launch_decode_instance<LPK, 4>(a, st);
+    else if (a.kv_group % 2 == 0) launch_decode_instance<LPK, 2>(a, st);
+    else launch_decode_instance<LPK, 1>(a, st);
+}
+
 int launch_decode_split(const FwdArgs& a, hipStream_t st)
 {
-    const unsigned groups = (unsigned)((long long)a.B * a.H * a.num_splits);
-    const bool alibi = a.alibi != nullptr;
-    if (a.d > 64) {
-        if (alibi) hipLaunchKernelGGL((decode_split_kernel<16, true>), dim3(groups), dim3(256), 0, st, a);
-        else hipLaunchKernelGGL((decode_split_kernel<16, false>), dim3(groups), dim3(256), 0, st, a);
-    } else if (a.d > 32) {
-        if (alibi) hipLaunchKernelGGL((decode_split_kernel<8, true>), dim3(groups), dim3(256), 0, st, a);
-        else hipLaunchKernelGGL((decode_split_kernel<8, false>), dim3(groups), dim3(256), 0, st, a);
-    } else {
-        if (alibi) hipLaunchKernelGGL((decode_split_kernel<4, true>), dim3(groups), dim3(256), 0, st, a);
-        else hipLaunchKernelGGL((decode_split_kernel<4, false>), dim3(groups), dim3(256), 0, st, a);
-    }
+    if (a.d > 64) launch_decode_bucket<16>(a, st);
+    else if (a.d > 32) launch_decode_bucket<8>(a, st);
+    else launch_decode_bucket<4>(a, st);
     return (int)hipGetLastError();
 }
 

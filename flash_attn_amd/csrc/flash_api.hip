@@ -39,6 +39,7 @@ int validate_shape(const flash_params* p, bool* empty)
     if (!(p->dropout_p >= 0.0f && p->dropout_p < 1.0f)) return FLASH_EINVAL;
     if (p->num_splits > FLASH_MAX_SPLITS) return FLASH_ESPLITS;
     if ((long long)p->B * p->H > 0x7fffffffLL / 2) return FLASH_EINVAL;
+    if (p->H_kv < 0 || (p->H_kv > 0 && (p->H_kv > p->H || p->H % p->H_kv != 0))) return FLASH_EINVAL;
     if (p->B == 0 || p->H == 0 || p->Nq == 0) *empty = true;
     return FLASH_OK;
 }
@@ -77,6 +78,8 @@ void fill_args(const flash_params* p, int splits, fa::FwdArgs* a)
     a->Nq = p->Nq;
     a->Nk = p->Nk;
     a->d = p->d;
+    a->Hk = p->H_kv > 0 ? p->H_kv : (p->H > 0 ? p->H : 1);
+    a->kv_group = p->H > 0 ? p->H / a->Hk : 1;
     a->causal = p->is_causal ? 1 : 0;
     a->wl = p->window_left;
     a->wr = p->window_right;

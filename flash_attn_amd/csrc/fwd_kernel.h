@@ -45,7 +45,6 @@ struct FwdCfg {
     static constexpr int VBUF = BC * SV;
     static constexpr int SMEM = 2 * KBUF + 2 * VBUF;
     static constexpr int NLD = BC * CH / 256;  // 16-byte chunks per thread per tile (K and V each)
-    static constexpr bool kPipelined = false;  // issue S(t+1) = K(t+1) Q^T next to softmax(S(t)); costs 32*NB registers
     static_assert(D % 32 == 0 && D <= 128, "head-dim bucket");
     static_assert((BC * CH) % 256 == 0, "tile chunks must divide over the group");
 };
@@ -165,8 +164,9 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
     }
 
     const half_t* __restrict__ Qbh = a.Q + (size_t)bh * Nq * d;
-    const half_t* __restrict__ Kbh = a.K + (size_t)bh * Nk * d;
-    const half_t* __restrict__ Vbh = a.V + (size_t)bh * Nk * d;
+    const int kvs = a.kv_slice(bh);
+    const half_t* __restrict__ Kbh = a.K + (size_t)kvs * Nk * d;
+    const half_t* __restrict__ Vbh = a.V + (size_t)kvs * Nk * d;
 
     // ---- Q fragments (B operand of S^T = K Q^T): lane holds row l32, columns 16*ks + 8*g .. +7
     v8h qf[NB][KS];
@@ -369,76 +369,34 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
             for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[nb][ks]));
     };
 
-    if constexpr (!C::kPipelined) {
-        // ---- plain double-buffered loop: tile t+1 is fetched from global memory while tile t is computed.
-        if (ntiles > 0) {
-            gload(Kbh, tile_begin, kreg);
-            gload(Vbh, tile_begin, vreg);
-            put_k(0);
-            put_v(0);
+    // ---- double-buffered loop: tile t+1 is fetched from global memory while tile t is computed
+    if (ntiles > 0) {
+        gload(Kbh, tile_begin, kreg);
+        gload(Vbh, tile_begin, vreg);
+        put_k(0);
+        put_v(0);
+    }
+    pin_q();
+    __syncthreads();
+    for (int t = 0; t < ntiles; ++t) {
+        const int cur = t & 1;
+        const int kb0 = (tile_begin + t) * BC;
+        const bool has1 = t + 1 < ntiles;
+        if (has1) {
+            gload(Kbh, tile_begin + t + 1, kreg);
+            gload(Vbh, tile_begin + t + 1, vreg);
         }
-        pin_q();
+        v16f s[2][NB];
+        v8h pf[2][2][NB];
+        qk(cur, s);
+        const bool need_mask = (kb0 < lo_max) || (kb0 + BC - 1 > hi_min);
+        softmax(need_mask, kb0, s, pf);
+        pv(cur, pf);
+        if (has1) {
+            put_k(cur ^ 1);
+            put_v(cur ^ 1);
+        }
         __syncthreads();
-        for (int t = 0; t < ntiles; ++t) {
-            const int cur = t & 1;
-            const int kb0 = (tile_begin + t) * BC;
-            const bool has1 = t + 1 < ntiles;
-            if (has1) {
-                gload(Kbh, tile_begin + t + 1, kreg);
-                gload(Vbh, tile_begin + t + 1, vreg);
-            }
-            v16f s[2][NB];
-            v8h pf[2][2][NB];
-            qk(cur, s);
-            const bool need_mask = (kb0 < lo_max) || (kb0 + BC - 1 > hi_min);
-            softmax(need_mask, kb0, s, pf);
-            pv(cur, pf);
-            if (has1) {
-                put_k(cur ^ 1);
-                put_v(cur ^ 1);
-            }
-            __syncthreads();
-        }
-    } else {
-        // ---- software pipeline.  Iteration t works on tile t: S(t) was produced one iteration earlier, so the
-        // MFMAs of S(t+1) = K(t+1) Q^T are issued next to the VALU work of softmax(S(t)), followed by O += P(t) V(t).
-        // LDS: K(t+1) in K buffer (t+1)&1, V(t) in V buffer t&1; the global loads of K(t+2) and V(t+1) fly meanwhile
-        // and are written to the freed buffers before the single barrier of the iteration.
-        v16f s_cur[2][NB];
-        if (ntiles > 0) {
-            gload(Kbh, tile_begin, kreg);
-            gload(Vbh, tile_begin, vreg);
-            put_k(0);
-            put_v(0);
-            if (ntiles > 1) {
-                gload(Kbh, tile_begin + 1, kreg);
-                put_k(1);
-            }
-        }
-        pin_q();
-        __syncthreads();
-        if (ntiles > 0) qk(0, s_cur);
-        for (int t = 0; t < ntiles; ++t) {
-            const int kb0 = (tile_begin + t) * BC;
-            const bool has1 = t + 1 < ntiles, has2 = t + 2 < ntiles;
-            if (has2) gload(Kbh, tile_begin + t + 2, kreg);
-            if (has1) gload(Vbh, tile_begin + t + 1, vreg);
-            const bool need_mask = (kb0 < lo_max) || (kb0 + BC - 1 > hi_min);
-            v8h pf[2][2][NB];
-            v16f s_next[2][NB];
-            if (has1) qk((t + 1) & 1, s_next);
-            softmax(need_mask, kb0, s_cur, pf);
-            pv(t & 1, pf);
-            if (has2) put_k(t & 1);
-            if (has1) put_v((t + 1) & 1);
-            __syncthreads();
-            if (has1) {
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int nb = 0; nb < NB; ++nb) s_cur[kb][nb] = s_next[kb][nb];
-            }
-        }
     }
 
     // ---------------- epilogue: normalise once, store O (fp16) + LSE, or the fp32 split partials

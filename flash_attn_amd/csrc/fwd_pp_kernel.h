@@ -163,8 +163,9 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     }
 
     const half_t* __restrict__ Qbh = a.Q + (size_t)bh * Nq * d;
-    const half_t* __restrict__ Kbh = a.K + (size_t)bh * Nk * d;
-    const half_t* __restrict__ Vbh = a.V + (size_t)bh * Nk * d;
+    const int kvs = a.kv_slice(bh);
+    const half_t* __restrict__ Kbh = a.K + (size_t)kvs * Nk * d;
+    const half_t* __restrict__ Vbh = a.V + (size_t)kvs * Nk * d;
 
     // ---- Q fragments
     v8h qf[KS];

@@ -37,7 +37,7 @@ enum {
 
 /* Superset of mykernelParamType (include/utils.h:21-44).
  *   reference field            here
- *   Q,K,V (half*)              Q,K,V            fp16 [B,H,Nq|Nk,d] contiguous, same layout
+ *   Q,K,V (half*)              Q,K,V            fp16 [B,H,Nq|Nk,d] contiguous, same layout (K,V: [B,H_kv,Nk,d] if H_kv is set)
  *   O (float*)                 O                fp16 [B,H,Nq,d]  (the reference stores fp32)
  *   --                         LSE              fp32 [B,H,Nq]    natural-log sum-exp of the masked scaled scores
  *   O_tmp, L, M                O_partial, LSE_partial   fp32 [B,H,S,Nq,d] and [B,H,S,Nq]; LSE_s = M_s + log L_s
@@ -73,6 +73,10 @@ typedef struct flash_params {
      * applied to every in-range (i, j) as one byte (1 = kept) into keep_mask_out [B,H,Nq,Nk].  No counterpart in
      * the reference, whose dropout is never verified (src/main.cu:44,222). */
     uint8_t *keep_mask_out;
+    /* Number of K/V heads (grouped-query / multi-query attention): K and V are [B,H_kv,Nk,d] and query head h reads
+     * K/V head h / (H / H_kv).  0 means H (one K/V head per query head, all the reference can express: it indexes
+     * K and V with the query head, src/flash_forward.h:57-59).  H must be a multiple of H_kv. */
+    int H_kv;
 } flash_params;
 
 /* Tiled forward over the whole key range: replaces

@@ -84,6 +84,9 @@ def test_argument_errors_are_codes_not_aborts(fa):
         assert entry(C.byref(_params(fa, dropout_p=float("nan"))), None) == E_INVAL
         assert entry(C.byref(_params(fa, softmax_scale=float("inf"))), None) == E_INVAL
         assert entry(C.byref(_params(fa, num_splits=129)), None) == E_SPLITS
+        assert entry(C.byref(_params(fa, H=6, H_kv=4)), None) == E_INVAL  # query heads must be a multiple of K/V heads
+        assert entry(C.byref(_params(fa, H=2, H_kv=4)), None) == E_INVAL
+        assert entry(C.byref(_params(fa, H=2, H_kv=-1)), None) == E_INVAL
         # empty problems are a no-op
         assert entry(C.byref(_params(fa, B=0)), None) == 0
         assert entry(C.byref(_params(fa, Nq=0, Q=None, O=None, LSE=None)), None) == 0
