@@ -179,53 +179,40 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         }
     }
 
-    // ---- direct global -> LDS tile loads.  Block `blk` of a K stage is the fragment (ks = blk / 2, kb = blk % 2):
-    // lane l holds row 32 kb + l % 32, columns 16 ks + 8 (l / 32) .. +7.  KiB `q` of a V stage holds the two transpose-read
-    // blocks tb = 2 q, 2 q + 1, tb = (st * MB + mb) * 2 + h: 16-lane group G of a block holds keys
-    // 16 st + 8 h + 4 (G / 2) + 0..3, columns 32 mb + 16 (G % 2) + 0..15, four keys x 32 bytes in lane order.
-    // Wave w fetches blocks w, w + 8, ...; offsets are bytes from the slice base for the first tile of the group.
-    uint32_t kgo[NKL], vgo[NVL];
-    int vkey[NVL];
-#pragma unroll
-    for (int x = 0; x < NKL; ++x) {
-        const int blk = wave + 8 * x;
-        const int row = 32 * (blk & 1) + l32;
-        kgo[x] = (uint32_t)(((tile_begin * BC + row) * d + 16 * (blk >> 1) + 8 * g) * 2);
-    }
-#pragma unroll
-    for (int x = 0; x < NVL; ++x) {
-        const int tb = 2 * (wave + 8 * x) + g;
-        const int st = tb / (2 * MB), mb = (tb >> 1) % MB, hh = tb & 1;
-        const int j = lane & 31, G = j >> 3, u = j & 7;
-        vkey[x] = 16 * st + 8 * hh + 4 * (G >> 1) + (u >> 1);
-        vgo[x] = (uint32_t)(((tile_begin * BC + vkey[x]) * d + 32 * mb + 16 * (G & 1) + 8 * (u & 1)) * 2);
+    // ---- direct global -> LDS tile loads.  A stage holds its 64-key tile row-major (256 bytes per key) with the
+    // 16-byte chunks of a row permuted, so that the requests of a wave are whole consecutive rows (four per KiB: the
+    // memory pipeline serves those 2.4x faster than 16-byte pieces of 32 different rows) and the fragment reads stay
+    // free of bank conflicts:
+    //   K: chunk c of key r sits in slot c ^ (r % 16)   -> ds_read_b128 of 16 keys x one chunk covers all 64 banks
+    //   V: 32-byte chunk c of key r sits in slot c ^ sigma(r), sigma(r) = 2 (r % 4) + (r / 4) % 2
+    //                                                  -> a transpose read of 4 keys x 2 chunks x 2 lane groups does
+    // KiB block x of a stage = keys 4x .. 4x+3; wave w requests blocks w and w + 8, lane i the 16 bytes of slot i % 16
+    // of key 4x + i / 16.  Offsets are bytes from the slice base for the first tile of the group.
+    static_assert(D == 128, "tile layout below: 16 chunks of 16 bytes per key");
+    const int dkey = 4 * wave + (lane >> 4);  // key of this lane in block w; + 32 in block w + 8
+    uint32_t kgo, vgo;
+    {
+        const int slot = lane & 15;
+        const int sigma = 2 * (dkey & 3) + ((dkey >> 2) & 1);
+        kgo = (uint32_t)((tile_begin * BC + dkey) * d * 2 + ((slot ^ (dkey & 15)) << 4));
+        vgo = (uint32_t)((tile_begin * BC + dkey) * d * 2 + ((((slot >> 1) ^ sigma) << 5) | ((slot & 1) << 4)));
     }
     const char* const Kb = reinterpret_cast<const char*>(Kbh);
     const char* const Vb = reinterpret_cast<const char*>(Vbh);
-    // tile index t counts from tile_begin; rows past Nk re-read row Nk - 1 (their scores are masked)
-    auto load_k = [&](int t, FA_LDS char* stage) {
-        const uint32_t toff = (uint32_t)t * (uint32_t)(BC * d * 2);
+    // tile index t counts from tile_begin; keys past Nk re-read key Nk - 1 (their scores are masked)
+    auto load_tile = [&](const char* base, uint32_t go, int t, FA_LDS char* stage) {
         const int rows_left = Nk - (tile_begin + t) * BC;  // >= 1
 #pragma unroll
         for (int x = 0; x < NKL; ++x) {
-            uint32_t o = kgo[x] + toff;
-            if (rows_left < BC) {
-                const int row = 32 * ((wave + 8 * x) & 1) + l32;
-                if (row >= rows_left) o -= (uint32_t)((row - rows_left + 1) * d * 2);
-            }
-            dma_kib(Kb, o, stage + (wave + 8 * x) * 1024);
+            const int key = dkey + 32 * x;
+            uint32_t o = go + (uint32_t)t * (uint32_t)(BC * d * 2) + (uint32_t)(32 * x * d * 2);
+            if (rows_left < BC && key >= rows_left) o -= (uint32_t)((key - rows_left + 1) * d * 2);
+            dma_kib(base, o, stage + (wave + 8 * x) * 1024);
         }
     };
-    auto load_v = [&](int t, FA_LDS char* stage) {
-        const uint32_t toff = (uint32_t)t * (uint32_t)(BC * d * 2);
-        const int rows_left = Nk - (tile_begin + t) * BC;
-#pragma unroll
-        for (int x = 0; x < NVL; ++x) {
-            uint32_t o = vgo[x] + toff;
-            if (rows_left < BC && vkey[x] >= rows_left) o -= (uint32_t)((vkey[x] - rows_left + 1) * d * 2);
-            dma_kib(Vb, o, stage + (wave + 8 * x) * 1024);
-        }
-    };
+    static_assert(NKL == NVL, "K and V tiles have the same shape");
+    auto load_k = [&](int t, FA_LDS char* stage) { load_tile(Kb, kgo, t, stage); };
+    auto load_v = [&](int t, FA_LDS char* stage) { load_tile(Vb, vgo, t, stage); };
 
     // ---- accumulators
     v16f oacc[MB];
@@ -239,8 +226,16 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     float slope2 = 0.0f;
     if constexpr (kAlibi) slope2 = a.alibi ? a.alibi[h] * kLog2e : 0.0f;
 
-    const int k_rd = lane * 16;  // fragment-major: a fragment is read back in lane order
-    const int v_rd = lane * 8;
+    // Lane parts of the fragment addresses (layout above).  K fragment (ks, kb): key 32 kb + l32, chunk 2 ks + g
+    // -> k_rd ^ (32 ks) + 8192 kb.  V transpose read (st, mb, half h) of lane (G = lane / 16, e = lane / 4 % 4,
+    // j = lane % 4): key 16 st + 8 h + 4 (G / 2) + e, 32-byte chunk 2 mb + G % 2, bytes 8 j .. 8 j + 7
+    // -> v_rd ^ (64 mb) + 4096 st + 2048 h.
+    const int k_rd = l32 * 256 + ((g ^ (l32 & 1)) << 4) + (((l32 & 15) >> 1) << 5);
+    int v_rd;
+    {
+        const int G = lane >> 4, e = (lane >> 2) & 3, j = lane & 3;
+        v_rd = (4 * (G >> 1) + e) * 256 + (((G & 1) ^ (G >> 1)) << 5) + 8 * j + (e << 6);
+    }
 
     v16f s[2];
     v8h pf[2][2];
@@ -254,23 +249,26 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     VF vf[4][MB];
     constexpr int KPD = KS < 3 ? KS : 3;  // K k-steps in flight
     v8h kf[KS][2];
-    auto v_read = [&](FA_LDS const char* vbase, int st) {
+    // vbase / kbase: stage address + lane part, as an integer (the stage bases are multiples of 16 KiB, so the
+    // exclusive-or only touches the lane part)
+    auto lds_ptr = [](uint32_t addr) { return reinterpret_cast<FA_LDS const char*>(static_cast<uintptr_t>(addr)); };
+    auto v_read = [&](uint32_t vbase, int st) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
-            FA_LDS const char* p0 = vbase + (st * MB + mb) * 1024;
+            FA_LDS const char* p0 = lds_ptr(vbase ^ (uint32_t)(mb << 6)) + st * 4096;
             vf[st][mb].p[0] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((FA_LDS v4hp*)(p0));
-            vf[st][mb].p[1] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((FA_LDS v4hp*)(p0 + 512));
+            vf[st][mb].p[1] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((FA_LDS v4hp*)(p0 + 2048));
         }
     };
-    auto k_read = [&](FA_LDS const char* kbase, int ks) {
+    auto k_read = [&](uint32_t kbase, int ks) {
+        FA_LDS const char* p0 = lds_ptr(kbase ^ (uint32_t)(ks << 5));
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) kf[ks][kb] = *reinterpret_cast<FA_LDS const v8h*>(kbase + (2 * ks + kb) * 1024);
+        for (int kb = 0; kb < 2; ++kb) kf[ks][kb] = *reinterpret_cast<FA_LDS const v8h*>(p0 + kb * 8192);
     };
-    // Lane offset inside a fragment block.  It is laundered through an empty asm once per phase: the compiler would
-    // otherwise pre-add it to every per-fragment constant and keep one address register per read, instead of one base
-    // register plus the DS offset field.  (The stage pointers themselves must stay visible: they carry the
-    // no-alias information that separates these reads from the LDS-DMA writes in flight.)
-    auto lane_off = [&](int v) {
+    // Stage address + lane part of a fragment address.  The sum is laundered through an empty asm once per phase: the
+    // compiler would otherwise precompute every per-fragment address across iterations and keep one register per read.
+    auto frag_base = [&](FA_LDS const char* stage, int lane_part) {
+        uint32_t v = (uint32_t)(uintptr_t)stage + (uint32_t)lane_part;
         asm volatile("" : "+v"(v));
         return v;
     };
@@ -291,7 +289,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     };
     // stand-alone S^T = K Q^T (prologue only)
     auto qk = [&](FA_LDS const char* __restrict__ rdk) {
-        FA_LDS const char* kbase = rdk + lane_off(k_rd);
+        const uint32_t kbase = frag_base(rdk, k_rd);
 #pragma unroll
         for (int ks = 0; ks < KPD; ++ks) k_read(kbase, ks);
         s_clear();
@@ -304,7 +302,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     // MFMA phase body after the barrier: O += P V(t) with the first K(t+1) fragments fetched under its last MFMAs,
     // then S = K(t+1) Q^T.  One basic block, so that the read / MFMA interleaving below can be pinned.  After the last
     // tile the K stage holds stale data and the resulting S is never used (one wasted QK per row block).
-    auto mfma_phase = [&](FA_LDS const char* vbase, FA_LDS const char* kbase) {
+    auto mfma_phase = [&](uint32_t vbase, uint32_t kbase) {
         pv_mfma(0);
         __builtin_amdgcn_sched_barrier(0);  // step 0 first: its fragments were requested first
         v_read(vbase, 2);
@@ -424,8 +422,8 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         const bool need_mask = (kb0 < lo_max) || (kb0 + BC - 1 > hi_min);
         softmax(need_mask, kb0);
         __builtin_amdgcn_sched_barrier(0);
-        FA_LDS const char* vbase = rdv + lane_off(v_rd);
-        FA_LDS const char* kbase = rdk + lane_off(k_rd);
+        const uint32_t vbase = frag_base(rdv, v_rd);
+        const uint32_t kbase = frag_base(rdk, k_rd);
         v_read(vbase, 0);
         __builtin_amdgcn_sched_barrier(0);  // keep the request order: step 0 is consumed first
         v_read(vbase, 1);
