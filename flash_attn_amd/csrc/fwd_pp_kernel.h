@@ -33,7 +33,8 @@ struct PPCfg {
     static constexpr int KBUF = BC * D * 2;   // bytes per K stage (fragment-major, unpadded)
     static constexpr int VBUF = BC * D * 2;
     static constexpr int NST = 4;             // LDS stages per tensor
-    static constexpr int SMEM = NST * (KBUF + VBUF);
+    static constexpr int XBUF = 16 * 1024;    // with the stages that are empty at start: 8 KiB per wave for its Q rows
+    static constexpr int SMEM = NST * (KBUF + VBUF) + XBUF;
     static constexpr int NKL = (2 * KS) / 8;  // 1 KiB K blocks loaded per wave per tile
     static constexpr int NVL = (4 * MB) / 8;  // 1 KiB V blocks loaded per wave per tile
     static_assert(D == 64 || D == 128, "ping-pong kernel: head dim 64 or 128");
@@ -85,6 +86,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     extern __shared__ __attribute__((aligned(16))) char smem[];
     FA_LDS char* const Ks = (FA_LDS char*)smem;
     FA_LDS char* const Vs = Ks + NST * C::KBUF;
+    FA_LDS char* const Xs = Vs + NST * C::VBUF;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -167,17 +169,8 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     const half_t* __restrict__ Kbh = a.K + (size_t)kvs * Nk * d;
     const half_t* __restrict__ Vbh = a.V + (size_t)kvs * Nk * d;
 
-    // ---- Q fragments
+    // ---- Q fragments: fetched through LDS in the prologue below
     v8h qf[KS];
-    {
-        const half_t* qrow = Qbh + (size_t)(row_i < Nq ? row_i : Nq - 1) * d;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            union { v4u u; v8h h; } t;
-            t.u = *reinterpret_cast<const v4u*>(qrow + 16 * ks + 8 * g);
-            qf[ks] = t.h;
-        }
-    }
 
     // ---- direct global -> LDS tile loads.  A stage holds its 64-key tile row-major (256 bytes per key) with the
     // 16-byte chunks of a row permuted, so that the requests of a wave are whole consecutive rows (four per KiB: the
@@ -436,20 +429,43 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         lds_barrier();
     };
 
-    // ---- prologue: K(0..2), V(0..1) requested; everything landed before the first barrier
-    if (ntiles > 0) {
-        load_k(0, Ks);
-        load_v(0, Vs);
-        if (ntiles > 1) {
-            load_k(1, Ks + C::KBUF);
-            load_v(1, Vs + C::VBUF);
+    // ---- prologue: Q, K(0..2), V(0..1) requested; everything landed before the first barrier.
+    // Q takes the same route as the tiles (whole rows per request, chunk c of row r in slot c ^ (r % 16)): each wave
+    // stages its own 32 rows in 8 KiB of LDS that no tile uses before the first loop iteration, and reads its eight
+    // B-operand fragments back from there.  Private to the wave: only its own vmcnt wait stands between the two.
+    {
+        FA_LDS char* const qst = wave < 2   ? Xs + wave * 8192
+                                 : wave < 4 ? Vs + 2 * C::VBUF + (wave - 2) * 8192
+                                 : wave < 6 ? Ks + 3 * C::KBUF + (wave - 4) * 8192
+                                            : Vs + 3 * C::VBUF + (wave - 6) * 8192;
+        static_assert(C::XBUF == 2 * 8192 && C::KBUF == 2 * 8192 && C::VBUF == 2 * 8192 && C::NST == 4, "Q staging map");
+        const char* const Qb = reinterpret_cast<const char*>(Qbh);
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            const int rl = 4 * x + (lane >> 4);  // row of the wave's 32
+            const int gi = q0 + rblk * 32 + rl;
+            const uint32_t off = (uint32_t)((gi < Nq ? gi : Nq - 1) * d * 2 + (((lane & 15) ^ (rl & 15)) << 4));
+            dma_kib(Qb, off, qst + x * 1024);
         }
-        if (ntiles > 2) load_k(2, Ks + 2 * C::KBUF);
+        if (ntiles > 0) {
+            load_k(0, Ks);
+            load_v(0, Vs);
+            if (ntiles > 1) {
+                load_k(1, Ks + C::KBUF);
+                load_v(1, Vs + C::VBUF);
+            }
+            if (ntiles > 2) load_k(2, Ks + 2 * C::KBUF);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (a memory clobber: the reads below stay below)
+        const uint32_t qbase = (uint32_t)(uintptr_t)qst + (uint32_t)k_rd;  // same lane part as a K fragment
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+            qf[ks] = *reinterpret_cast<FA_LDS const v8h*>(
+                reinterpret_cast<FA_LDS const char*>(static_cast<uintptr_t>(qbase ^ (uint32_t)(ks << 5))));
     }
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));  // Q has landed: no vmcnt waits on qf in the loop
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    lds_barrier();
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));  // Q is in registers before the loop
+    lds_barrier();  // tiles visible to all waves; every wave has read its Q rows (their LDS is reused by the loop)
     if (ntiles > 0) qk(Ks);
     if (grp == 1) lds_barrier();  // second wave group runs half an iteration behind
 
@@ -482,8 +498,8 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         const float l = xhalf_sum(l_run);
         const float inv = l > 0.0f ? 1.0f / l : 0.0f;
         const float lse = l > 0.0f ? (m_ref + fast_log2(l)) * kLn2 : -INFINITY;
-        if (row_i < Nq) {
-            if (a.num_splits > 1) {
+        if (a.num_splits > 1) {
+            if (row_i < Nq) {
                 const size_t prow = ((size_t)bh * a.num_splits + split) * Nq + row_i;
                 if (g == 0) a.LSE_partial[prow] = lse;
                 float* op = a.O_partial + prow * d;
@@ -496,18 +512,30 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
                                  oacc[mb][4 * rg + 3] * inv};
                         *reinterpret_cast<v4f*>(op + dc) = o;
                     }
-            } else {
-                if (g == 0) a.LSE[(size_t)bh * Nq + row_i] = lse;
-                half_t* op = a.O + ((size_t)bh * Nq + row_i) * d;
+            }
+        } else {
+            if (row_i < Nq && g == 0) a.LSE[(size_t)bh * Nq + row_i] = lse;
+            // O: a lane holds 4 consecutive head-dim columns of one row at a time; written like that, a wave store
+            // would touch 32 rows x 8 bytes.  The wave's 32 x 128 fp16 block is turned round in 8 KiB of LDS instead
+            // (all tile reads of the work-group are behind the last barrier; chunk c of row r in slot c ^ (r % 16), as
+            // for the tiles), and leaves as four whole rows per store instruction.
+            FA_LDS char* const ost = Ks + wave * 8192;
 #pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
+            for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                    for (int rg = 0; rg < 4; ++rg) {
-                        const int dc = 32 * mb + 8 * rg + 4 * g;
-                        v4h o = {(half_t)(oacc[mb][4 * rg] * inv), (half_t)(oacc[mb][4 * rg + 1] * inv),
-                                 (half_t)(oacc[mb][4 * rg + 2] * inv), (half_t)(oacc[mb][4 * rg + 3] * inv)};
-                        *reinterpret_cast<v4h*>(op + dc) = o;
-                    }
+                for (int rg = 0; rg < 4; ++rg) {
+                    v4h o = {(half_t)(oacc[mb][4 * rg] * inv), (half_t)(oacc[mb][4 * rg + 1] * inv),
+                             (half_t)(oacc[mb][4 * rg + 2] * inv), (half_t)(oacc[mb][4 * rg + 3] * inv)};
+                    const int slot = (4 * mb + rg) ^ (l32 & 15);
+                    *reinterpret_cast<FA_LDS v4h*>(ost + l32 * 256 + slot * 16 + g * 8) = o;
+                }
+            char* const Ob = reinterpret_cast<char*>(a.O + (size_t)bh * Nq * d);
+#pragma unroll
+            for (int x = 0; x < 8; ++x) {
+                const int rl = 4 * x + (lane >> 4);
+                const int gi = q0 + rblk * 32 + rl;
+                const v4u val = *reinterpret_cast<FA_LDS const v4u*>(ost + x * 1024 + lane * 16);
+                if (gi < Nq) *reinterpret_cast<v4u*>(Ob + (size_t)gi * d * 2 + (((lane & 15) ^ (rl & 15)) << 4)) = val;
             }
         }
     }
