@@ -430,24 +430,52 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
                 }
         } else {
             if (g == 0) a.LSE[(size_t)bh * Nq + i] = lse;
-            half_t* op = a.O + ((size_t)bh * Nq + i) * d;
+            if constexpr (!kVec) {
+                half_t* op = a.O + ((size_t)bh * Nq + i) * d;
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
+                for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                for (int rg = 0; rg < 4; ++rg) {
-                    const int dc = 32 * mb + 8 * rg + 4 * g;
-                    if (kVec) {
-                        if (kFullD || dc < d) {
-                            v4h o = {(half_t)(oacc[mb][nb][4 * rg] * inv), (half_t)(oacc[mb][nb][4 * rg + 1] * inv),
-                                     (half_t)(oacc[mb][nb][4 * rg + 2] * inv), (half_t)(oacc[mb][nb][4 * rg + 3] * inv)};
-                            *reinterpret_cast<v4h*>(op + dc) = o;
-                        }
-                    } else {
+                    for (int rg = 0; rg < 4; ++rg) {
+                        const int dc = 32 * mb + 8 * rg + 4 * g;
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
                             if (dc + e < d) op[dc + e] = (half_t)(oacc[mb][nb][4 * rg + e] * inv);
                     }
-                }
+            }
+        }
+    }
+    if constexpr (kVec) {
+        if (a.num_splits == 1) {
+            // O of the vector path: a lane holds 4 consecutive head-dim columns of one row at a time, which as a direct
+            // store would be 32 rows x 8 bytes per instruction.  The wave's 32 x d block goes through LDS instead (the tile
+            // buffers are free behind the last barrier; rows padded by 16 bytes) and leaves in consecutive 16-byte pieces
+            // of whole rows.
+            constexpr int SO = 2 * D + 16;
+            static_assert(4 * NB * 32 * SO <= C::SMEM, "O staging fits the tile buffers");
+            char* const ost = smem + wave * (NB * 32 * SO);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const float l = xhalf_sum(l_run[nb]);
+                const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int rg = 0; rg < 4; ++rg) {
+                        v4h o = {(half_t)(oacc[mb][nb][4 * rg] * inv), (half_t)(oacc[mb][nb][4 * rg + 1] * inv),
+                                 (half_t)(oacc[mb][nb][4 * rg + 2] * inv), (half_t)(oacc[mb][nb][4 * rg + 3] * inv)};
+                        *reinterpret_cast<v4h*>(ost + (nb * 32 + l32) * SO + (32 * mb + 8 * rg + 4 * g) * 2) = o;
+                    }
+            }
+            char* const Ob = reinterpret_cast<char*>(a.O + (size_t)bh * Nq * d);
+            constexpr int NP = NB * 32 * CH;  // 16-byte pieces of the wave's block, CH per row
+#pragma unroll
+            for (int p0 = 0; p0 < NP; p0 += 64) {
+                const int p = p0 + lane;
+                const int rl = p / CH, ch = p % CH;
+                const int gi = q0 + wave * C::RW + rl;
+                if (p < NP && gi < Nq && (kFullD || ch * 8 < d))
+                    *reinterpret_cast<v4u*>(Ob + (size_t)gi * d * 2 + ch * 16) = *reinterpret_cast<const v4u*>(ost + rl * SO + ch * 16);
+            }
         }
     }
 }
