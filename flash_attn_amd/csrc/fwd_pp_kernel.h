@@ -1,4 +1,4 @@
-// Ping-pong variant of the tiled forward kernel for head dims 64 and 128 that fill their bucket (d == D).
+// Ping-pong variant of the tiled forward kernel for head dim 128 (d == D == 128).
 //
 // Same math as fwd_kernel.h (S^T = K Q^T and O^T += V^T P^T on MFMA 32x32x16, Q in registers, online softmax per
 // lane, 64-key tiles).  What changes is the schedule and the way tiles reach LDS:
@@ -10,10 +10,11 @@
 //    phase while the other is in its VALU phase.  (Two independent 4-wave groups per CU do not interleave this way
 //    by themselves: measured MFMA / VALU co-execution was 11 % of the time.)
 //  * Tiles go from global memory straight into LDS (global_load_lds_dwordx4: 64 lanes write one contiguous KiB, each
-//    lane fetching from its own global address), in a fragment-major layout: the KiB written by one load is exactly
-//    what the 64 lanes of one ds_read_b128 (K fragment) or of two ds_read_b64_tr_b16 (V fragment halves) read back
-//    as base + lane * 16 (resp. * 8).  No staging registers, no ds_write, no padding, conflict-free by construction,
-//    and every LDS read address is one base register plus an immediate.
+//    lane fetching 16 bytes from its own global address): no staging registers, no ds_write.  A stage holds its tile
+//    row-major with the 16-byte chunks of every row permuted (exclusive-or with low bits of the row number), so that
+//    a request covers four whole rows of global memory and the fragment reads (ds_read_b128 for K, ds_read_b64_tr_b16
+//    for V) are free of bank conflicts; a fragment address is one base register ^ constant plus an immediate.
+//    Q and O go through 8 KiB of wave-private LDS in the same layout, for the same reason (whole rows per request).
 //  * Four LDS stages per tensor: K(t+3) and V(t+2) are requested at the start of the VALU phase of iteration t and
 //    waited for (vmcnt) at the end of the MFMA phase of the same iteration; with the half-iteration offset their
 //    slots (K(t-1), V(t-2)) were last read two barriers earlier, and the first reader comes two barriers later.
@@ -30,7 +31,7 @@ struct PPCfg {
     static constexpr int BC = 64;             // keys per tile
     static constexpr int KS = D / 16;
     static constexpr int MB = D / 32;
-    static constexpr int KBUF = BC * D * 2;   // bytes per K stage (fragment-major, unpadded)
+    static constexpr int KBUF = BC * D * 2;   // bytes per K stage (row-major, permuted chunks, no padding)
     static constexpr int VBUF = BC * D * 2;
     static constexpr int NST = 4;             // LDS stages per tensor
     static constexpr int XBUF = 16 * 1024;    // with the stages that are empty at start: 8 KiB per wave for its Q rows
