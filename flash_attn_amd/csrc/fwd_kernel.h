@@ -449,7 +449,8 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
             // O of the vector path: a lane holds 4 consecutive head-dim columns of one row at a time, which as a direct
             // store would be 32 rows x 8 bytes per instruction.  The wave's 32 x d block goes through LDS instead (the tile
             // buffers are free behind the last barrier; rows padded by 16 bytes) and leaves in consecutive 16-byte pieces
-            // of whole rows.
+            // of whole rows.  The stores are non-temporal: O is not read again by this launch, and lines left dirty in L2
+            // would only be written back when the kernel ends.
             constexpr int SO = 2 * D + 16;
             static_assert(4 * NB * 32 * SO <= C::SMEM, "O staging fits the tile buffers");
             char* const ost = smem + wave * (NB * 32 * SO);
@@ -474,7 +475,8 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
                 const int rl = p / CH, ch = p % CH;
                 const int gi = q0 + wave * C::RW + rl;
                 if (p < NP && gi < Nq && (kFullD || ch * 8 < d))
-                    *reinterpret_cast<v4u*>(Ob + (size_t)gi * d * 2 + ch * 16) = *reinterpret_cast<const v4u*>(ost + rl * SO + ch * 16);
+                    __builtin_nontemporal_store(*reinterpret_cast<const v4u*>(ost + rl * SO + ch * 16),
+                                                reinterpret_cast<v4u*>(Ob + (size_t)gi * d * 2 + ch * 16));
             }
         }
     }

@@ -519,7 +519,8 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
             // O: a lane holds 4 consecutive head-dim columns of one row at a time; written like that, a wave store
             // would touch 32 rows x 8 bytes.  The wave's 32 x 128 fp16 block is turned round in 8 KiB of LDS instead
             // (all tile reads of the work-group are behind the last barrier; chunk c of row r in slot c ^ (r % 16), as
-            // for the tiles), and leaves as four whole rows per store instruction.
+            // for the tiles), and leaves as four whole rows per store instruction (non-temporal: O is not read again by this
+            // launch, and lines left dirty in L2 would only be written back when the kernel ends).
             FA_LDS char* const ost = Ks + wave * 8192;
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
@@ -536,7 +537,8 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
                 const int rl = 4 * x + (lane >> 4);
                 const int gi = q0 + rblk * 32 + rl;
                 const v4u val = *reinterpret_cast<FA_LDS const v4u*>(ost + x * 1024 + lane * 16);
-                if (gi < Nq) *reinterpret_cast<v4u*>(Ob + (size_t)gi * d * 2 + (((lane & 15) ^ (rl & 15)) << 4)) = val;
+                if (gi < Nq)
+                    __builtin_nontemporal_store(val, reinterpret_cast<v4u*>(Ob + (size_t)gi * d * 2 + (((lane & 15) ^ (rl & 15)) << 4)));
             }
         }
     }
