@@ -70,12 +70,23 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 // Philox4x32-10.  Dropout contract: key = (lo32(seed), hi32(seed)); counter = (j >> 2, i, b*H + h, lo32(offset));
 // element (i, j) uses output word j & 3 and is kept iff word >= floor(p * 2^32).  Replaces the stateful
 // curandStatePhilox4_32_10_t draw of the reference (src/flash_forward.h:50-54,227).
+// 32 x 32 -> 64-bit product in one instruction (v_mad_u64_u32; integer multiplies run at a quarter of the VALU rate,
+// and the compiler would issue two of them, v_mul_hi_u32 and v_mul_lo_u32, per product)
+__device__ __forceinline__ void mul_wide_u32(uint32_t m, uint32_t x, uint32_t& hi, uint32_t& lo)
+{
+    uint64_t r;
+    asm("v_mad_u64_u32 %0, vcc, %1, %2, 0" : "=v"(r) : "s"(m), "v"(x) : "vcc");
+    hi = (uint32_t)(r >> 32);
+    lo = (uint32_t)r;
+}
+
 __device__ __forceinline__ v4u philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1)
 {
 #pragma unroll
     for (int r = 0; r < 10; ++r) {
-        const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
-        const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+        uint32_t hi0, lo0, hi1, lo1;
+        mul_wide_u32(0xD2511F53u, c0, hi0, lo0);
+        mul_wide_u32(0xCD9E8D57u, c2, hi1, lo1);
         c0 = hi1 ^ c1 ^ k0;
         c1 = lo1;
         c2 = hi0 ^ c3 ^ k1;
