@@ -152,11 +152,24 @@ FLASH_EXPORT int flash_forward_splitkv(const flash_params* p, void* stream)
     fa::FwdArgs a;
     fill_args(p, splits, &a);
     int e;
-    // one query row per head, 16-byte rows, no dropout: bandwidth-bound streaming kernel; otherwise the tiled kernel
-    if (p->Nq == 1 && p->d % 8 == 0 && p->dropout_p == 0.0f && p->softmax_scale > 0.0f)
-        e = record_hip(fa::launch_decode_split(a, st));
-    else
+    if (p->Nq == 1 && a.kv_group >= 4 && !p->alibi_slopes && p->window_left < 0 && p->dropout_p == 0.0f) {
+        // Decode with grouped K/V heads: the G query heads of one K/V head, one row each, are the G rows of one
+        // attention problem over that K/V head -- Q [B,H,1,d] is [B,H_kv,G,d] in memory, and so are O, LSE and the
+        // split workspace, and no mask depends on the row.  The tiled kernel then streams K/V once per K/V head and
+        // does the arithmetic on the MFMA units (measured 1.4x - 4x faster than G dot products per key on the VALU
+        // for G = 8 ... 32, equal at G = 4).
+        a.H = a.Hk;
+        a.Nq = a.kv_group;
+        a.kv_group = 1;
+        a.causal = 0;
+        a.Tr = (a.Nq + kRowsPerGroup - 1) / kRowsPerGroup;
         e = launch_tiled(p, a, st);
+    } else if (p->Nq == 1 && p->d % 8 == 0 && p->dropout_p == 0.0f && p->softmax_scale > 0.0f) {
+        // one query row per head, 16-byte rows, no dropout: bandwidth-bound streaming kernel
+        e = record_hip(fa::launch_decode_split(a, st));
+    } else {
+        e = launch_tiled(p, a, st);
+    }
     if (e != FLASH_OK || splits == 1) return e;
     return record_hip(fa::launch_combine(a, st));
 }

@@ -378,6 +378,9 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
     }
     pin_q();
     __syncthreads();
+    // A wave whose rows all lie past Nq (fewer than 128 query rows: short prompts, or the heads of one K/V head decoding
+    // together) only helps to stage the tiles.
+    const bool wave_live = q0 + wave * C::RW < Nq;
     for (int t = 0; t < ntiles; ++t) {
         const int cur = t & 1;
         const int kb0 = (tile_begin + t) * BC;
@@ -386,12 +389,14 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
             gload(Kbh, tile_begin + t + 1, kreg);
             gload(Vbh, tile_begin + t + 1, vreg);
         }
-        v16f s[2][NB];
-        v8h pf[2][2][NB];
-        qk(cur, s);
-        const bool need_mask = (kb0 < lo_max) || (kb0 + BC - 1 > hi_min);
-        softmax(need_mask, kb0, s, pf);
-        pv(cur, pf);
+        if (wave_live) {
+            v16f s[2][NB];
+            v8h pf[2][2][NB];
+            qk(cur, s);
+            const bool need_mask = (kb0 < lo_max) || (kb0 + BC - 1 > hi_min);
+            softmax(need_mask, kb0, s, pf);
+            pv(cur, pf);
+        }
         if (has1) {
             put_k(cur ^ 1);
             put_v(cur ^ 1);

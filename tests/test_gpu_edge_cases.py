@@ -181,6 +181,10 @@ def test_grouped_query_heads(fa, oracle, H, Hk, Nq, Nk, d, kw):
     (6, 2, 128, 777, dict()),                         # 3 per group: falls back to one query head per work-group
     (32, 2, 96, 2100, dict(alibi=True)),              # 16 per group: two work-groups of 8
     (4, 1, 128, 5000, dict(causal=True)),             # multi-query
+    (32, 2, 128, 2500, dict()),                       # 16 per group, no row-dependent mask: tiled kernel, heads as rows
+    (32, 1, 64, 1111, dict()),                        # 32 per group
+    (8, 2, 72, 900, dict()),                          # head dim not a bucket width
+    (12, 2, 31, 700, dict()),                         # 6 per group, odd head dim
 ])
 def test_grouped_query_decode(fa, oracle, H, Hk, d, Nk, kw):
     B = 2
