@@ -98,4 +98,19 @@ __device__ __forceinline__ v4u philox4x32_10(uint32_t c0, uint32_t c1, uint32_t 
     return o;
 }
 
+// Raises the dynamic-LDS limit of a kernel once per device (the attribute belongs to the device's copy of the kernel).
+// `done` is the caller's per-kernel flag array; concurrent first calls may both set the attribute, which is harmless.
+constexpr int kMaxDevices = 64;
+inline hipError_t ensure_dynamic_lds(const void* kern, int bytes, bool (&done)[kMaxDevices])
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) dev = kMaxDevices - 1;  // beyond the table: set it on every launch
+    if (done[dev] && dev != kMaxDevices - 1) return hipSuccess;
+    e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) done[dev] = true;
+    return e;
+}
+
 }  // namespace fa

@@ -499,13 +499,8 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
 {
     using C = FwdCfg<D, NB>;
     auto kern = fwd_kernel<D, NB, VAR>;
-    static bool attr_done = false;  // per instantiation
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+    static bool attr_done[kMaxDevices] = {};  // per instantiation and device
+    if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), C::SMEM, attr_done); e != hipSuccess) return e;
     const long long groups = (long long)a.Tr * a.B * a.H * a.num_splits;
     hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(256), C::SMEM, st, a);
     return hipGetLastError();

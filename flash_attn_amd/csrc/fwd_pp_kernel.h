@@ -549,13 +549,8 @@ inline hipError_t launch_fwd_pp_instance(const FwdArgs& a, hipStream_t st)
 {
     using C = PPCfg<D>;
     auto kern = fwd_pp_kernel<D, VAR>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+    static bool attr_done[kMaxDevices] = {};  // per instantiation and device
+    if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), C::SMEM, attr_done); e != hipSuccess) return e;
     FwdArgs b = a;
     b.Tr = (a.Nq + C::BR - 1) / C::BR;
     const long long groups = (long long)b.Tr * a.B * a.H * a.num_splits;
