@@ -147,19 +147,22 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
         hi[nb] = h_;
         iif[nb] = (float)ii;
     }
-    // wave-uniform bounds for the "does this tile need the element test" decision
-    int lo_max, hi_min;
+    // wave-uniform bounds: [lo_max, hi_min] is visible to every row of the wave (a tile inside it needs no element
+    // test), nothing outside [lo_min, hi_max] is visible to any of them (a tile outside it is skipped by the wave)
+    int lo_max, hi_min, lo_min, hi_max;
     {
         const int first = q0 + wave * C::RW, last = first + C::RW - 1;
         const int iif_ = (first < Nq ? first : Nq - 1) + shift, iil_ = (last < Nq ? last : Nq - 1) + shift;
-        lo_max = 0;
-        hi_min = Nk - 1;
-        if (a.wl >= 0) lo_max = max(0, iil_ - a.wl);
-        if (a.causal) hi_min = min(hi_min, iif_);
-        if (a.wr >= 0) hi_min = min(hi_min, iif_ + a.wr);
+        lo_max = lo_min = 0;
+        hi_min = hi_max = Nk - 1;
+        if (a.wl >= 0) lo_max = max(0, iil_ - a.wl), lo_min = max(0, iif_ - a.wl);
+        if (a.causal) hi_min = min(hi_min, iif_), hi_max = min(hi_max, iil_);
+        if (a.wr >= 0) hi_min = min(hi_min, iif_ + a.wr), hi_max = min(hi_max, iil_ + a.wr);
         if (a.num_splits > 1) {
             lo_max = max(lo_max, kmin);
+            lo_min = max(lo_min, kmin);
             hi_min = min(hi_min, kmax - 1);
+            hi_max = min(hi_max, kmax - 1);
         }
     }
 
@@ -379,7 +382,8 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
     pin_q();
     __syncthreads();
     // A wave whose rows all lie past Nq (fewer than 128 query rows: short prompts, or the heads of one K/V head decoding
-    // together) only helps to stage the tiles.
+    // together) only helps to stage the tiles, and so does any wave for a tile that none of its rows can see (the far
+    // end of the causal diagonal block, the near end of a sliding window).
     const bool wave_live = q0 + wave * C::RW < Nq;
     for (int t = 0; t < ntiles; ++t) {
         const int cur = t & 1;
@@ -389,7 +393,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
             gload(Kbh, tile_begin + t + 1, kreg);
             gload(Vbh, tile_begin + t + 1, vreg);
         }
-        if (wave_live) {
+        if (wave_live && kb0 <= hi_max && kb0 + BC - 1 >= lo_min) {
             v16f s[2][NB];
             v8h pf[2][2][NB];
             qk(cur, s);

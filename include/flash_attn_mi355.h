@@ -70,8 +70,9 @@ typedef struct flash_params {
     uint64_t offset;
     int num_splits;
     /* Optional debug output: when non-NULL and dropout_p > 0, the forward kernel also stores the keep decision it
-     * applied to every in-range (i, j) as one byte (1 = kept) into keep_mask_out [B,H,Nq,Nk].  No counterpart in
-     * the reference, whose dropout is never verified (src/main.cu:44,222). */
+     * applied to (i, j) as one byte (1 = kept) into keep_mask_out [B,H,Nq,Nk], for every (i, j) that the masks leave
+     * visible; the bytes of masked-out pairs may or may not be written.  No counterpart in the reference, whose
+     * dropout is never verified (src/main.cu:44,222). */
     uint8_t *keep_mask_out;
     /* Number of K/V heads (grouped-query / multi-query attention): K and V are [B,H_kv,Nk,d] and query head h reads
      * K/V head h / (H / H_kv).  0 means H (one K/V head per query head, all the reference can express: it indexes
