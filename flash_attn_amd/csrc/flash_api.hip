@@ -97,9 +97,9 @@ void fill_args(const flash_params* p, int splits, fa::FwdArgs* a)
 
 int launch_tiled(const flash_params* p, const fa::FwdArgs& a, hipStream_t st)
 {
-    int variant = (p->d % 8 == 0) ? 1 : 0;
-    // a non-positive scale does not commute with the row maximum: take the variant that scales first
-    if (p->alibi_slopes || !(p->softmax_scale > 0.0f)) variant |= 2;
+    // A non-positive scale does not commute with the row maximum: only the element-wise instance scales first.
+    int variant = (p->d % 8 == 0 && p->softmax_scale > 0.0f) ? 1 : 0;
+    if (p->alibi_slopes) variant |= 2;
     if (p->dropout_p > 0.0f) variant |= 4;
     int e;
     if (p->d <= 32) e = fa::launch_fwd_d32(a, variant, 1, st);

@@ -24,6 +24,7 @@
 //    element-wise load / store path (kVec = false).
 #pragma once
 #include "common.h"
+#include <cstdlib>
 
 namespace fa {
 
@@ -38,9 +39,12 @@ struct FwdCfg {
     static constexpr int CH = D / 8;          // 16-byte chunks per row
     // LDS row strides in bytes.  K rows are read 16 bytes per lane by 32 consecutive rows: stride/16 odd spreads
     // them over all banks.  V rows are read by ds_read_b64_tr_b16, four consecutive rows of 64 bytes per half
-    // wave: stride = 64 (mod 128) puts the four rows on disjoint bank groups.
+    // wave: a stride of 64 (mod 128) puts the four rows on disjoint bank groups.
     static constexpr int SK = D * 2 + 16;
-    static constexpr int SV = ((D * 2) % 128 == 64) ? D * 2 : D * 2 + 64;
+    static constexpr int SV = D * 2;
+    // Where the row length is a multiple of 128 bytes, the two 64-byte halves of each 128 bytes are exchanged in rows
+    // 2, 3 (mod 4), which has the same effect without padding.
+    static constexpr bool VSWZ = (D * 2) % 128 == 0;
     static constexpr int KBUF = BC * SK;
     static constexpr int VBUF = BC * SV;
     static constexpr int SMEM = 2 * KBUF + 2 * VBUF;
@@ -82,7 +86,7 @@ constexpr float kLazyTau = 8.0f;
 constexpr int kVarVec = 1, kVarAlibi = 2, kVarDropout = 4, kVarFullD = 8;
 
 template <int D, int NB, int VAR>
-__global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs a)
+__global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 0 ? 3 : 2) : 1) fwd_kernel(const FwdArgs a)
 {
     constexpr bool kVec = (VAR & kVarVec) != 0, kAlibi = (VAR & kVarAlibi) != 0, kDropout = (VAR & kVarDropout) != 0,
                    kFullD = (VAR & kVarFullD) != 0;
@@ -210,7 +214,8 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
     auto put_v = [&](int buf) {
 #pragma unroll
         for (int x = 0; x < NLD; ++x)
-            *reinterpret_cast<v4u*>(Vs + buf * C::VBUF + ld_row[x] * SV + ld_col[x] * 2) = vreg[x];
+            *reinterpret_cast<v4u*>(Vs + buf * C::VBUF + ld_row[x] * SV +
+                                    ((ld_col[x] * 2) ^ (C::VSWZ ? ((ld_row[x] >> 1) & 1) << 6 : 0))) = vreg[x];
     };
 
     // ---- accumulators
@@ -226,13 +231,23 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
             for (int r = 0; r < 16; ++r) oacc[mb][nb][r] = 0.0f;
     }
 
+    // Scores leave the MFMA unscaled.  With a positive scale the scaling commutes with the row maximum and is folded
+    // into the exponent (one fma per score): cs = scale, and the ALiBi bias is added beforehand divided by the scale.
+    // A non-positive scale is served by the element-wise instance alone (the host sends it there): then the scores are
+    // scaled first and cs = 1.
     const float c2 = a.scale_log2;
-    float slope2 = 0.0f;
-    if constexpr (kAlibi) slope2 = a.alibi ? a.alibi[h] * kLog2e : 0.0f;
+    const bool scale_late = kVec || c2 > 0.0f;
+    const float cs = scale_late ? c2 : 1.0f;
+    float slope2 = 0.0f, nsig = 0.0f;
+    if constexpr (kAlibi) {
+        slope2 = a.alibi ? a.alibi[h] * kLog2e : 0.0f;
+        nsig = scale_late ? -slope2 / c2 : 0.0f;
+    }
 
     // LDS read offsets of this lane
     const int k_rd = l32 * SK + g * 16;                                          // + kb*32*SK + ks*32
     const int v_rd = (4 * g + ((lane & 15) >> 2)) * SV + (((lane >> 4) & 1) * 16 + (lane & 3) * 4) * 2;  // + row/col blocks
+    const int v_sw = C::VSWZ ? ((lane >> 3) & 1) << 6 : 0;
 
     // S^T = K Q^T of the tile in K buffer `buf`
     auto qk = [&](int buf, v16f (&s)[2][NB]) {
@@ -256,32 +271,55 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
     };
 
     // online softmax of one tile (per query row = per lane); leaves P^T packed to fp16 in pf
-    auto softmax = [&](bool need_mask, int kb0, v16f (&s)[2][NB], v8h (&pf)[2][2][NB]) {
+    // mask_sides: bit 0 = some row of the wave has its first allowed key inside or after this tile, bit 1 = some row
+    // has its last allowed key inside or before it (both wave-uniform)
+    auto softmax = [&](int mask_sides, int kb0, v16f (&s)[2][NB], v8h (&pf)[2][2][NB]) {
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             if constexpr (kAlibi) {
                 // score*scale - slope*|i - j|  (src/main.cu:315,324), in the log2 domain
                 const float jb = (float)(kb0 + 4 * g) - iif[nb];
+                if (scale_late) {
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                    for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const float dist = jb + (float)(32 * kb + 8 * (r >> 2) + (r & 3));
-                        s[kb][nb][r] = s[kb][nb][r] * c2 - slope2 * __builtin_fabsf(dist);
-                    }
+                        for (int r = 0; r < 16; ++r)
+                            s[kb][nb][r] = __builtin_fmaf(nsig, __builtin_fabsf(jb + (float)(32 * kb + 8 * (r >> 2) + (r & 3))), s[kb][nb][r]);
+                } else {
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                            s[kb][nb][r] = s[kb][nb][r] * c2 - slope2 * __builtin_fabsf(jb + (float)(32 * kb + 8 * (r >> 2) + (r & 3)));
+                }
             }
-            if (need_mask) {
-                // wave-uniform and rare (boundary tiles only).  Routing the bounds through an empty volatile asm keeps
-                // this a real branch: otherwise the compiler folds the block into selects that every tile executes.
+            if (mask_sides != 0) {
+                // Wave-uniform and rare (boundary tiles only).  Routing the bounds through an empty volatile asm keeps
+                // these real branches: otherwise the compiler folds the blocks into selects that every tile executes.
+                // A tile that only one end of the interval crosses takes one comparison per score.
                 int lo_rel = lo[nb] - kb0 - 4 * g, hi_rel = hi[nb] - kb0 - 4 * g;
                 asm volatile("; boundary tile: element mask" : "+v"(lo_rel), "+v"(hi_rel));
+                if (mask_sides == 1) {
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                    for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int jr = 32 * kb + 8 * (r >> 2) + (r & 3);
-                        if (jr < lo_rel || jr > hi_rel) s[kb][nb][r] = -INFINITY;
-                    }
+                        for (int r = 0; r < 16; ++r)
+                            if (32 * kb + 8 * (r >> 2) + (r & 3) < lo_rel) s[kb][nb][r] = -INFINITY;
+                } else if (mask_sides == 2) {
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                            if (32 * kb + 8 * (r >> 2) + (r & 3) > hi_rel) s[kb][nb][r] = -INFINITY;
+                } else {
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const int jr = 32 * kb + 8 * (r >> 2) + (r & 3);
+                            if (jr < lo_rel || jr > hi_rel) s[kb][nb][r] = -INFINITY;
+                        }
+                }
             }
             float mx = -INFINITY;
 #pragma unroll
@@ -289,7 +327,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
 #pragma unroll
                 for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kb][nb][r]);
             mx = xhalf_max(mx);
-            if constexpr (!kAlibi) mx *= c2;  // host guarantees scale > 0 here: max commutes with the scaling
+            mx *= cs;  // cs > 0
             if (__builtin_amdgcn_ballot_w64(mx > m_ref[nb] + kLazyTau) != 0ull) {
                 const float m_new = fmaxf(m_ref[nb], mx);
                 float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_ref[nb] - m_new);
@@ -307,9 +345,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    float p;
-                    if constexpr (kAlibi) p = fast_exp2(s[kb][nb][r] - m_use);
-                    else p = fast_exp2(__builtin_fmaf(s[kb][nb][r], c2, -m_use));
+                    const float p = fast_exp2(__builtin_fmaf(s[kb][nb][r], cs, -m_use));
                     rs += p;
                     s[kb][nb][r] = p;
                 }
@@ -343,14 +379,16 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
 
     // O^T += V^T P^T with the tile in V buffer `buf`
     auto pv = [&](int buf, v8h (&pf)[2][2][NB]) {
-        const char* vbase = Vs + buf * C::VBUF + v_rd;
+        // (a lane's rows all share bit 1 of the row index: the swizzle is one per-lane choice between two bases)
+        const char* const vb[2] = {Vs + buf * C::VBUF + v_rd + v_sw, Vs + buf * C::VBUF + v_rd + (v_sw ^ (C::VSWZ ? 64 : 0))};
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt) {
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {
-                    const char* p0 = vbase + (32 * kb + 16 * tt) * SV + mb * 64;
+                    const char* p0 = C::VSWZ ? vb[mb & 1] + (32 * kb + 16 * tt) * SV + (mb >> 1) * 128
+                                             : vb[0] + (32 * kb + 16 * tt) * SV + mb * 64;
                     union { v4hp p[2]; v8h v; } af;
                     af.p[0] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((FA_LDS v4hp*)(p0));
                     af.p[1] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((FA_LDS v4hp*)(p0 + 8 * SV));
@@ -397,8 +435,8 @@ __global__ void __launch_bounds__(256, NB == 1 ? 2 : 1) fwd_kernel(const FwdArgs
             v16f s[2][NB];
             v8h pf[2][2][NB];
             qk(cur, s);
-            const bool need_mask = (kb0 < lo_max) || (kb0 + BC - 1 > hi_min);
-            softmax(need_mask, kb0, s, pf);
+            const int mask_sides = (kb0 < lo_max ? 1 : 0) | (kb0 + BC - 1 > hi_min ? 2 : 0);
+            softmax(mask_sides, kb0, s, pf);
             pv(cur, pf);
         }
         if (has1) {
@@ -506,7 +544,9 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
     static bool attr_done[kMaxDevices] = {};  // per instantiation and device
     if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), C::SMEM, attr_done); e != hipSuccess) return e;
     const long long groups = (long long)a.Tr * a.B * a.H * a.num_splits;
-    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(256), C::SMEM, st, a);
+    static const int pad = getenv("FA_LDS_PAD") ? atoi(getenv("FA_LDS_PAD")) : 0;
+    if (pad) hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM + pad);
+    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(256), C::SMEM + pad, st, a);
     return hipGetLastError();
 }
 

@@ -216,9 +216,12 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[mb][r] = 0.0f;
 
-    const float c2 = a.scale_log2;
-    float slope2 = 0.0f;
-    if constexpr (kAlibi) slope2 = a.alibi ? a.alibi[h] * kLog2e : 0.0f;
+    // Scores leave the MFMA unscaled.  With a positive scale the scaling commutes with the row maximum and is folded
+    // into the exponent (one fma per score): cs = scale, and the ALiBi bias is added beforehand divided by the scale.
+    // (The host sends a non-positive scale to the element-wise instance of the 4-wave kernel.)
+    const float c2 = a.scale_log2, cs = c2;
+    float nsig = 0.0f;
+    if constexpr (kAlibi) nsig = a.alibi ? -(a.alibi[h] * kLog2e) / c2 : 0.0f;
 
     // Lane parts of the fragment addresses (layout above).  K fragment (ks, kb): key 32 kb + l32, chunk 2 ks + g
     // -> k_rd ^ (32 ks) + 8192 kb.  V transpose read (st, mb, half h) of lane (G = lane / 16, e = lane / 4 % 4,
@@ -327,27 +330,43 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     };
 
     // online softmax of the tile whose scores sit in s; leaves P^T packed to fp16 in pf
-    auto softmax = [&](bool need_mask, int kb0) {
+    // mask_sides: bit 0 = some row of the wave has its first allowed key inside or after this tile, bit 1 = some row has
+    // its last allowed key inside or before it (both wave-uniform)
+    auto softmax = [&](int mask_sides, int kb0) {
         if constexpr (kAlibi) {
+            // score*scale - slope*|i - j|  (src/main.cu:315,324), in the log2 domain
             const float jb = (float)(kb0 + 4 * g) - iif;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float dist = jb + (float)(32 * kb + 8 * (r >> 2) + (r & 3));
-                    s[kb][r] = s[kb][r] * c2 - slope2 * __builtin_fabsf(dist);
-                }
+                for (int r = 0; r < 16; ++r)
+                    s[kb][r] = __builtin_fmaf(nsig, __builtin_fabsf(jb + (float)(32 * kb + 8 * (r >> 2) + (r & 3))), s[kb][r]);
         }
-        if (need_mask) {
+        if (mask_sides != 0) {
+            // a tile that only one end of the interval crosses takes one comparison per score
             int lo_rel = lo - kb0 - 4 * g, hi_rel = hi - kb0 - 4 * g;
             asm volatile("; boundary tile: element mask" : "+v"(lo_rel), "+v"(hi_rel));
+            if (mask_sides == 1) {
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+                for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int jr = 32 * kb + 8 * (r >> 2) + (r & 3);
-                    if (jr < lo_rel || jr > hi_rel) s[kb][r] = -INFINITY;
-                }
+                    for (int r = 0; r < 16; ++r)
+                        if (32 * kb + 8 * (r >> 2) + (r & 3) < lo_rel) s[kb][r] = -INFINITY;
+            } else if (mask_sides == 2) {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        if (32 * kb + 8 * (r >> 2) + (r & 3) > hi_rel) s[kb][r] = -INFINITY;
+            } else {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int jr = 32 * kb + 8 * (r >> 2) + (r & 3);
+                        if (jr < lo_rel || jr > hi_rel) s[kb][r] = -INFINITY;
+                    }
+            }
         }
         float mx = -INFINITY;
 #pragma unroll
@@ -355,7 +374,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
 #pragma unroll
             for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kb][r]);
         mx = xhalf_max(mx);
-        if constexpr (!kAlibi) mx *= c2;
+        mx *= cs;  // cs > 0
         if (__builtin_amdgcn_ballot_w64(mx > m_ref + kLazyTau) != 0ull) {
             const float m_new = fmaxf(m_ref, mx);
             float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_ref - m_new);
@@ -373,9 +392,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                float p;
-                if constexpr (kAlibi) p = fast_exp2(s[kb][r] - m_use);
-                else p = fast_exp2(__builtin_fmaf(s[kb][r], c2, -m_use));
+                const float p = fast_exp2(__builtin_fmaf(s[kb][r], cs, -m_use));
                 rs += p;
                 s[kb][r] = p;
             }
@@ -413,8 +430,8 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         // ---------------- VALU phase: request the tiles to come, softmax of tile t
         if (t + 3 < ntiles) load_k(t + 3, wrk);
         if (t + 2 < ntiles) load_v(t + 2, wrv);
-        const bool need_mask = (kb0 < lo_max) || (kb0 + BC - 1 > hi_min);
-        softmax(need_mask, kb0);
+        const int mask_sides = (kb0 < lo_max ? 1 : 0) | (kb0 + BC - 1 > hi_min ? 2 : 0);
+        softmax(mask_sides, kb0);
         __builtin_amdgcn_sched_barrier(0);
         const uint32_t vbase = frag_base(rdv, v_rd);
         const uint32_t kbase = frag_base(rdk, k_rd);
