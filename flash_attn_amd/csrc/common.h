@@ -38,7 +38,7 @@ struct FwdArgs {
     int Hk, kv_group;    // K/V heads and query heads per K/V head (H = Hk * kv_group)
     int causal, wl, wr;  // wl / wr < 0: unbounded
     float scale_log2;    // softmax_scale * log2(e)
-    uint32_t drop_thr;   // keep iff philox word >= drop_thr
+    uint32_t drop_thr;   // keep iff 16-bit philox field >= drop_thr
     float drop_rscale;   // 1 / (1 - p)
     uint32_t seed_lo, seed_hi, off_lo;
     int num_splits;      // 1: write O/LSE; > 1: write the partial workspace
@@ -67,9 +67,14 @@ __device__ __forceinline__ float xhalf_sum(float v)
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-// Philox4x32-10.  Dropout contract: key = (lo32(seed), hi32(seed)); counter = (j >> 2, i, b*H + h, lo32(offset));
-// element (i, j) uses output word j & 3 and is kept iff word >= floor(p * 2^32).  Replaces the stateful
-// curandStatePhilox4_32_10_t draw of the reference (src/flash_forward.h:50-54,227).
+// Philox4x32-10.  Dropout contract: one call yields eight 16-bit fields (field f = bits 16*(f&1).. of output word f>>1)
+// and serves eight keys of one query row: key = (lo32(seed), hi32(seed)), counter = (call(j), i, b*H + h, lo32(offset)),
+// element (i, j) reads field(j) and is kept iff that field >= floor(p * 2^16).  Of every 16 consecutive keys the call
+// with even index serves keys 0-3 and 8-11, the odd one keys 4-7 and 12-15: the eight keys whose scores one lane of the
+// tiled kernels holds (32x32 MFMA accumulator layout), so that a lane uses every bit it computes.  Replaces the
+// stateful curandStatePhilox4_32_10_t draw of the reference (src/flash_forward.h:50-54,227).
+__host__ __device__ __forceinline__ uint32_t dropout_call(uint32_t j) { return 2u * (j >> 4) + ((j >> 2) & 1u); }
+__host__ __device__ __forceinline__ uint32_t dropout_field(uint32_t j) { return 4u * ((j >> 3) & 1u) + (j & 3u); }
 // 32 x 32 -> 64-bit product in one instruction (v_mad_u64_u32; integer multiplies run at a quarter of the VALU rate,
 // and the compiler would issue two of them, v_mul_hi_u32 and v_mul_lo_u32, per product)
 __device__ __forceinline__ void mul_wide_u32(uint32_t m, uint32_t x, uint32_t& hi, uint32_t& lo)
@@ -97,6 +102,9 @@ __device__ __forceinline__ v4u philox4x32_10(uint32_t c0, uint32_t c1, uint32_t 
     v4u o = {c0, c1, c2, c3};
     return o;
 }
+
+// 16-bit field f (0..7) of a Philox output
+__device__ __forceinline__ uint32_t philox_field16(const v4u& w, int f) { return (w[f >> 1] >> (16 * (f & 1))) & 0xffffu; }
 
 // Raises the dynamic-LDS limit of a kernel once per device (the attribute belongs to the device's copy of the kernel).
 // `done` is the caller's per-kernel flag array; concurrent first calls may both set the attribute, which is harmless.

@@ -221,22 +221,25 @@ __global__ void __launch_bounds__(256) combine_kernel(const float* __restrict__ 
     if (lane == 0) LSE[(size_t)bh * Nq + i] = sum > 0.0f ? mx + __logf(sum) : -INFINITY;
 }
 
-// keep[b,h,i,j] = philox word (j & 3) of counter (j >> 2, i, b*H + h, lo32(offset)) >= threshold
+// keep[b,h,i,j] = (16-bit field dropout_field(j) of the Philox call dropout_call(j) of row (b*H + h, i)) >= threshold;
+// one thread per call, i.e. per eight keys: 16*(c >> 1) + 8*r2 + 4*(c & 1) + e
 __global__ void __launch_bounds__(256) keep_mask_kernel(uint8_t* __restrict__ mask, long long rows, int Nq, int Nk,
                                                         uint32_t thr, uint32_t seed_lo, uint32_t seed_hi,
                                                         uint32_t off_lo)
 {
-    const int groups = (Nk + 3) >> 2;
-    const long long total = rows * groups;
+    const int calls = 2 * ((Nk + 15) >> 4);
+    const long long total = rows * calls;
     for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (long long)gridDim.x * 256) {
-        const long long r = idx / groups;
-        const int jg = (int)(idx % groups);
+        const long long r = idx / calls;
+        const int c = (int)(idx % calls);
         const uint32_t bh = (uint32_t)(r / Nq), i = (uint32_t)(r % Nq);
-        const v4u w = philox4x32_10((uint32_t)jg, i, bh, off_lo, seed_lo, seed_hi);
+        const v4u w = philox4x32_10((uint32_t)c, i, bh, off_lo, seed_lo, seed_hi);
         uint8_t* mrow = mask + (size_t)r * Nk;
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-            if (4 * jg + e < Nk) mrow[4 * jg + e] = w[e] >= thr ? 1 : 0;
+        for (int f = 0; f < 8; ++f) {
+            const int j = 16 * (c >> 1) + 8 * (f >> 2) + 4 * (c & 1) + (f & 3);
+            if (j < Nk) mrow[j] = philox_field16(w, f) >= thr ? 1 : 0;
+        }
     }
 }
 
@@ -279,7 +282,7 @@ int launch_keep_mask(uint8_t* mask, int B, int H, int Nq, int Nk, uint32_t thr, 
                      hipStream_t st)
 {
     const long long rows = (long long)B * H * Nq;
-    const long long total = rows * ((Nk + 3) / 4);
+    const long long total = rows * (2 * ((Nk + 15) / 16));  // one thread per Philox call
     long long groups = (total + 255) / 256;
     if (groups > 65536) groups = 65536;
     if (groups < 1) groups = 1;

@@ -221,9 +221,9 @@ FLASH_EXPORT int flash_num_splits_heuristic(int batch_nheads_mblocks, int num_SM
 
 FLASH_EXPORT uint32_t flash_dropout_threshold(float dropout_p)
 {
-    double t = std::floor((double)dropout_p * 4294967296.0);
+    double t = std::floor((double)dropout_p * 65536.0);
     if (!(t > 0.0)) t = 0.0;
-    if (t > 4294967295.0) t = 4294967295.0;
+    if (t > 65535.0) t = 65535.0;
     return (uint32_t)t;
 }
 

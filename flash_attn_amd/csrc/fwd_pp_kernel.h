@@ -403,14 +403,21 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int rg = 0; rg < 4; ++rg) {
-                    const int j0 = kb0 + 32 * kb + 8 * rg + 4 * g;
-                    const v4u w = philox4x32_10((uint32_t)(j0 >> 2), i_u, (uint32_t)bh, a.off_lo, a.seed_lo, a.seed_hi);
+                for (int q = 0; q < 2; ++q) {
+                    // the lane's eight keys among the 16 from jg on: field f belongs to key jg + 8*(f>>2) + 4*g + (f&3)
+                    const int jg = kb0 + 32 * kb + 16 * q;
+                    const v4u w = philox4x32_10(dropout_call((uint32_t)(jg + 4 * g)), i_u, (uint32_t)bh, a.off_lo, a.seed_lo, a.seed_hi);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const bool keep = w[e] >= a.drop_thr;
-                        s[kb][4 * rg + e] = keep ? s[kb][4 * rg + e] * a.drop_rscale : 0.0f;
-                        if (kout && row_i < Nq && j0 + e < Nk) kout[j0 + e] = keep ? 1 : 0;
+                    for (int f = 0; f < 8; ++f) {
+                        const int r = 8 * q + f;
+                        s[kb][r] = philox_field16(w, f) >= a.drop_thr ? s[kb][r] * a.drop_rscale : 0.0f;
+                    }
+                    if (a.keep_out != nullptr) {  // debug dump: one uniform branch per call, none per score
+#pragma unroll
+                        for (int f = 0; f < 8; ++f) {
+                            const int j = jg + 8 * (f >> 2) + 4 * g + (f & 3);
+                            if (row_i < Nq && j < Nk) kout[j] = philox_field16(w, f) >= a.drop_thr ? 1 : 0;
+                        }
                     }
                 }
         }

@@ -107,7 +107,11 @@ int flash_num_splits_heuristic(int batch_nheads_mblocks, int num_SMs, int num_n_
  * separately launched RNG step; the counter-based generator needs no state, so this only materialises the mask. */
 int flash_dropout_keep_mask(const flash_params *p, uint8_t *mask_out, void *stream);
 
-/* Integer drop threshold floor(p * 2^32) (host helper; element kept iff its Philox word >= threshold). */
+/* Integer drop threshold floor(p * 2^16), at most 65535 (host helper).  The dropout contract, reproducible on a CPU:
+ * Philox4x32-10 with key (lo32(seed), hi32(seed)) and counter (call(j), i, b*H + h, lo32(offset)), where
+ * call(j) = 2*(j >> 4) + ((j >> 2) & 1); the 128 output bits are eight 16-bit fields (field f = bits 16*(f & 1) and
+ * up of output word f >> 1), and element (i, j) is kept iff field 4*((j >> 3) & 1) + (j & 3) >= threshold.  Kept
+ * probabilities are scaled by 1/(1 - dropout_p); the row sum of the softmax is taken before the drop. */
 uint32_t flash_dropout_threshold(float dropout_p);
 
 /* Text of the last HIP error seen by this thread inside the library ("" if none). */

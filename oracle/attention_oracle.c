@@ -369,18 +369,21 @@ ORACLE_API void oracle_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2
     out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
 }
 
-/* Integer drop threshold: an element is kept iff its 32-bit word >= floor(p * 2^32).  This is the reference's rule
- * "drop iff uniform < p" (src/flash_forward.h:227-234) stated on the raw word, so that no float rounding enters. */
+/* Integer drop threshold: an element is kept iff its 16-bit random field >= floor(p * 2^16).  This is the reference's
+ * rule "drop iff uniform < p" (src/flash_forward.h:227-234) stated on raw bits, so that no float rounding enters. */
 ORACLE_API uint32_t oracle_dropout_threshold(float p)
 {
-    double t = floor((double)p * 4294967296.0);
-    if (t < 0.0) t = 0.0;
-    if (t > 4294967295.0) t = 4294967295.0;
+    double t = floor((double)p * 65536.0);
+    if (!(t > 0.0)) t = 0.0;
+    if (t > 65535.0) t = 65535.0;
     return (uint32_t)t;
 }
 
-/* Keep-mask of the device contract: key = (lo32(seed), hi32(seed)); counter = (j >> 2, i, b*H + h, lo32(offset));
- * element (i, j) reads output word j & 3.  mask [B,H,Nq,Nk] bytes, 1 = keep. */
+/* Keep-mask of the device contract.  One Philox call yields eight 16-bit fields (field f = bits 16*(f&1).. of output
+ * word f>>1) and serves eight keys of one query row: key = (lo32(seed), hi32(seed)), counter =
+ * (call(j), i, b*H + h, lo32(offset)) with call(j) = 2*(j >> 4) + ((j >> 2) & 1), and element (i, j) reads field
+ * 4*((j >> 3) & 1) + (j & 3).  (Of every 16 consecutive keys, the call with odd index serves keys 4-7 and 12-15: the
+ * eight keys whose scores one lane of the device kernel holds.)  mask [B,H,Nq,Nk] bytes, 1 = keep. */
 ORACLE_API void oracle_dropout_keep_mask(uint64_t seed, uint64_t offset, float p, int B, int H, int Nq, int Nk,
                                          uint8_t *mask, int nthreads)
 {
@@ -392,11 +395,16 @@ ORACLE_API void oracle_dropout_keep_mask(uint64_t seed, uint64_t offset, float p
     for (long long r = 0; r < rows; ++r) {
         const uint32_t bh = (uint32_t)(r / Nq), i = (uint32_t)(r % Nq);
         uint8_t *mrow = mask + (size_t)r * Nk;
-        for (int j4 = 0; j4 < Nk; j4 += 4) {
-            const uint32_t ctr[4] = {(uint32_t)(j4 >> 2), i, bh, (uint32_t)offset};
-            uint32_t w[4];
-            oracle_philox4x32_10(ctr, key, w);
-            for (int e = 0; e < 4 && j4 + e < Nk; ++e) mrow[j4 + e] = (uint8_t)(w[e] >= thr);
+        uint32_t have = 0xffffffffu, w[4] = {0, 0, 0, 0};
+        for (int j = 0; j < Nk; ++j) {
+            const uint32_t call = 2u * ((uint32_t)j >> 4) + (((uint32_t)j >> 2) & 1u);
+            const uint32_t f = 4u * (((uint32_t)j >> 3) & 1u) + ((uint32_t)j & 3u);
+            if (call != have) {
+                const uint32_t ctr[4] = {call, i, bh, (uint32_t)offset};
+                oracle_philox4x32_10(ctr, key, w);
+                have = call;
+            }
+            mrow[j] = (uint8_t)(((w[f >> 1] >> (16u * (f & 1u))) & 0xffffu) >= thr);
         }
     }
 }

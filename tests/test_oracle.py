@@ -186,16 +186,30 @@ def test_philox_against_independent_python(oracle):
 
 def test_dropout_threshold_and_mask_layout(oracle):
     assert oracle.dropout_threshold(0.0) == 0
-    assert oracle.dropout_threshold(0.5) == 2 ** 31
-    assert oracle.dropout_threshold(0.25) == 2 ** 30
-    assert oracle.dropout_threshold(0.1) == int(np.floor(float(np.float32(0.1)) * 2 ** 32))
-    B, H, Nq, Nk, p = 2, 3, 5, 11, 0.3
+    assert oracle.dropout_threshold(0.5) == 2 ** 15
+    assert oracle.dropout_threshold(0.25) == 2 ** 14
+    assert oracle.dropout_threshold(0.1) == int(np.floor(float(np.float32(0.1)) * 2 ** 16))
+    assert oracle.dropout_threshold(0.9999999) == 65535
+    B, H, Nq, Nk, p = 2, 3, 5, 43, 0.3
     seed, off = 0x1234567812345678, 9
     m = oracle.dropout_keep_mask(seed, off, p, B, H, Nq, Nk)
     thr = oracle.dropout_threshold(p)
-    for (b, h, i, j) in [(0, 0, 0, 0), (1, 2, 4, 10), (0, 1, 3, 7), (1, 0, 2, 5)]:
-        w = oracle.philox4x32_10([j >> 2, i, b * H + h, off], [seed & 0xFFFFFFFF, seed >> 32])[j & 3]
-        assert m[b, h, i, j] == (1 if w >= thr else 0)
+    # The contract restated call by call: call c of a row serves the keys 16*(c>>1) + 8*r + 4*(c&1) + e (r < 2, e < 4)
+    # with the 16-bit fields 4*r + e of the 128 output bits (word 0 lowest).  Every key is served exactly once.
+    want = np.full((B, H, Nq, Nk), 255, dtype=np.uint8)
+    for b in range(B):
+        for h in range(H):
+            for i in range(Nq):
+                for c in range(2 * ((Nk + 15) // 16)):
+                    w = oracle.philox4x32_10([c, i, b * H + h, off], [seed & 0xFFFFFFFF, seed >> 32])
+                    bits = w[0] | (w[1] << 32) | (w[2] << 64) | (w[3] << 96)
+                    for r in range(2):
+                        for e in range(4):
+                            jj = 16 * (c >> 1) + 8 * r + 4 * (c & 1) + e
+                            if jj < Nk:
+                                assert want[b, h, i, jj] == 255
+                                want[b, h, i, jj] = 1 if ((bits >> (16 * (4 * r + e))) & 0xFFFF) >= thr else 0
+    assert np.array_equal(m, want)
     assert oracle.dropout_keep_mask(1, 0, 0.0, 1, 1, 4, 9).all()
     big = oracle.dropout_keep_mask(1234, 0, 0.1, 1, 4, 256, 256)
     assert abs(big.mean() - 0.9) < 0.005
