@@ -72,7 +72,8 @@ DESCR = {
 }
 
 
-PROFILE_OF = {"cfg2": "fwd_kernel_d128_causal_prefill.md", "cfg5": "decode_split_kernel_d128_splitkv_decode.md"}
+PROFILE_OF = {"cfg2": "fwd_kernel_d128_causal_prefill.md", "cfg3": "fwd_kernel_d64_local_alibi.md",
+              "cfg4": "fwd_kernel_d96_causal_dropout.md", "cfg5": "decode_split_kernel_d128_splitkv_decode.md"}
 
 
 def measured_traffic(name):
