@@ -113,7 +113,21 @@ int resolve_splits(const flash_params* p)
 {
     const int n_blocks = (p->Nk + FLASH_SPLIT_KEY_GRANULE - 1) / FLASH_SPLIT_KEY_GRANULE;
     int s = p->num_splits;
-    if (s <= 0) {
+    if (s <= 0 && p->Nq == 1) {
+        // Decode streams K and V once and is bound by HBM: the reference's rule (fill the SMs once) leaves most of the
+        // bandwidth unused here, where one 256-thread work-group keeps far fewer bytes in flight than a CU can.
+        // Measured on 256 CUs, as long as a split still streams 512 keys or more: the one-row kernel keeps gaining up
+        // to about 32 work-groups per CU in the launch; the tiled kernel, which takes over when four or more query
+        // heads of a K/V head decode together (flash_forward_splitkv: one work-group per K/V head and split), is best
+        // near 2 per CU and loses 10-30 % beyond 8.
+        const int hk = p->H_kv > 0 ? p->H_kv : p->H;
+        const bool grouped = p->H / (hk > 0 ? hk : 1) >= 4;
+        const long long base = (long long)p->B * (grouped ? hk : p->H);
+        const long long target = (grouped ? 2LL : 32LL) * kNumCU;
+        const long long want = (target + base - 1) / (base > 0 ? base : 1);
+        const int by_keys = n_blocks / 4;  // 512 keys per split
+        s = (int)(want < by_keys ? want : by_keys);
+    } else if (s <= 0) {
         const int Tr = (p->Nq + kRowsPerGroup - 1) / kRowsPerGroup;
         // argument roles as in the reference's call (src/main.cu:125), with the CU count of the MI355X
         s = flash_num_splits_heuristic(Tr * p->H * p->B, kNumCU, n_blocks, FLASH_MAX_SPLITS, n_blocks * FLASH_SPLIT_KEY_GRANULE);

@@ -48,7 +48,7 @@ enum {
  *   --                         is_causal           (template bool Is_causal in the reference)
  *   alibi_slopes_ptr           alibi_slopes        fp32 [H] or NULL; score -= slope[h] * |i - j|
  *   dropout_prob, seed, states dropout_p, seed, offset   counter-based Philox4x32-10 instead of curand states
- *   split_num                  num_splits          (<= 0: flash_num_splits_heuristic with 256 CUs)
+ *   split_num                  num_splits          (<= 0: chosen by the library, see flash_forward_splitkv)
  * Row index used by masks and bias is i + (Nk - Nq), which is i whenever Nq == Nk (all the reference can express).
  */
 typedef struct flash_params {
@@ -89,7 +89,10 @@ int flash_forward(const flash_params *p, void *stream);
  *     forward_kernel_splitkv<...><<<dim3(Tr*split,H,B),256,smem>>>(param);
  *     forward_kernel_splitkv_combine<<<dim3(Tr,H,B),Br>>>(param);          (src/flash_forward_splitkv.h:14-16,347-348,
  *                                                                          src/main.cu:189-192)
- * Uses p->num_splits (heuristic when <= 0); needs the workspace when the resulting split count is > 1. */
+ * Uses p->num_splits; needs the workspace when the resulting split count is > 1.  With num_splits <= 0 the library
+ * chooses: flash_num_splits_heuristic with 256 CUs (the reference's rule, src/main.cu:125) for Nq > 1; for Nq == 1,
+ * which streams K and V once and is bound by memory bandwidth, enough splits of at least 512 keys to give every CU
+ * several work-groups.  flash_splitkv_resolve_splits returns the count either way. */
 int flash_forward_splitkv(const flash_params *p, void *stream);
 
 /* Bytes of O_partial and of LSE_partial needed for p (the cudaMallocs of src/main.cu:160-162). Either may be NULL. */

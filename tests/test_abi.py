@@ -120,10 +120,16 @@ def test_split_resolution_and_workspace(fa):
     assert fa.resolve_splits(1, 1, 128, 128, 64, 8) == 1
     assert fa.workspace_bytes(1, 1, 128, 128, 64, 8) == (0, 0)
     # heuristic (num_splits <= 0) with 256 CUs: the reference's checked-in shape B=1,H=8,N=1021 splits 4 ways,
-    # every benchmark shape stays unsplit
+    # the prefill benchmark shapes stay unsplit
     assert fa.resolve_splits(1, 8, 1021, 1021, 31, 0) == 4
     assert fa.resolve_splits(4, 16, 2048, 2048, 128, 0) == 1
-    assert fa.resolve_splits(16, 32, 1, 16384, 128, 0) == 1
+    # one query row (decode, bandwidth-bound): about 32 work-groups per CU, 512 keys or more per split
+    assert fa.resolve_splits(16, 32, 1, 16384, 128, 0) == 16
+    assert fa.resolve_splits(1, 32, 1, 16384, 128, 0) == 32
+    assert fa.resolve_splits(1, 32, 1, 2048, 128, 0) == 4
+    assert fa.resolve_splits(1, 8, 1, 1 << 20, 128, 0) == 128
+    assert fa.resolve_splits(512, 32, 1, 16384, 128, 0) == 1
+    assert fa.resolve_splits(1, 1, 1, 300, 64, 0) == 1
     with pytest.raises(fa.FlashError):
         fa.resolve_splits(1, 1, 1, 128, 64, 1000)
 
