@@ -260,3 +260,43 @@ def test_full_size_properties_decode(fa):
         assert torch.allclose(lS, l16, atol=2e-5)
     o, _ = fa.flash_forward_splitkv(q, k, torch.full_like(v, 0.5), num_splits=16)
     assert torch.allclose(o.float(), torch.full_like(o, 0.5, dtype=torch.float32), atol=1e-3)
+
+
+# The 8-wave kernel serves d = 128 with more than 1024 causal rows (or more than 128 rows without a causal mask):
+# ragged lengths beyond that threshold, Nq != Nk in both directions, every mask, grouped heads, dropout, split mode.
+@pytest.mark.parametrize("Nq,Nk,Hk,kw", [
+    (1100, 1100, 2, dict(causal=True)),
+    (1100, 1333, 2, dict(causal=True)),
+    (1333, 1100, 2, dict(causal=True)),                       # leading rows see no key: O = 0, LSE = -inf
+    (1100, 1100, 1, dict(causal=True)),                       # two query heads per K/V head
+    (1100, 1100, 2, dict(causal=True, window=(600, -1))),
+    (1100, 1100, 2, dict(causal=True, alibi=True)),
+    (1061, 1061, 2, dict(causal=True, dropout_p=0.2, seed=99, offset=5)),
+    (300, 1500, 2, dict(window=(700, 900))),
+])
+def test_eight_wave_kernel_cases(fa, oracle, Nq, Nk, Hk, kw):
+    import torch
+    B, H, d = 1, 2, 128
+    q = randn_f16_gpu((B, H, Nq, d), 21)
+    k = randn_f16_gpu((B, Hk, Nk, d), 22)
+    v = randn_f16_gpu((B, Hk, Nk, d), 23)
+    kr, vr = (t.repeat_interleave(H // Hk, dim=1).contiguous() for t in (k, v))
+    kw = dict(kw)
+    okw = {x: kw[x] for x in ("causal", "window") if x in kw}
+    if kw.pop("alibi", False):
+        sl, sl_t = _slopes(oracle, H)
+        kw["alibi_slopes"], okw["slopes"] = sl_t, sl
+    p = kw.get("dropout_p", 0.0)
+    if p > 0.0:
+        keep = oracle.dropout_keep_mask(kw["seed"], kw["offset"], p, B, H, Nq, Nk)
+        okw.update(keep_mask=torch.from_numpy(keep), p_drop=p)
+        o, lse, km = fa.flash_forward(q, k, v, return_keep_mask=True, **kw)
+        vis = np.tril(np.ones((Nq, Nk), dtype=bool), Nk - Nq)
+        assert np.array_equal(km.cpu().numpy()[..., vis], keep[..., vis])
+    else:
+        o, lse = fa.flash_forward(q, k, v, **kw)
+    O, L = oracle_forward_batched(oracle, q, kr, vr, **okw)
+    check_o_lse(o, lse, O, L, f"8-wave Nq={Nq} Nk={Nk} {sorted(kw)}")
+    if p == 0.0:
+        o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=3, **kw)
+        check_o_lse(o, lse, O, L, f"8-wave split Nq={Nq} Nk={Nk} {sorted(kw)}")
