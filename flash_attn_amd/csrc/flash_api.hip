@@ -128,8 +128,11 @@ int resolve_splits(const flash_params* p)
         const int by_keys = n_blocks / 4;  // 512 keys per split
         s = (int)(want < by_keys ? want : by_keys);
     } else if (s <= 0) {
-        const int Tr = (p->Nq + kRowsPerGroup - 1) / kRowsPerGroup;
-        // argument roles as in the reference's call (src/main.cu:125), with the CU count of the MI355X
+        const bool vec = p->d % 8 == 0 && p->softmax_scale > 0.0f;
+        const int rows = fa::fwd_uses_pingpong(p->d, vec, p->Nq, p->is_causal, p->window_left, p->window_right) ? 256 : kRowsPerGroup;
+        const int Tr = (p->Nq + rows - 1) / rows;
+        // argument roles as in the reference's call (src/main.cu:125), with the CU count of the MI355X and the row
+        // blocks of the kernel that will run
         s = flash_num_splits_heuristic(Tr * p->H * p->B, kNumCU, n_blocks, FLASH_MAX_SPLITS, n_blocks * FLASH_SPLIT_KEY_GRANULE);
     }
     if (s > n_blocks) s = n_blocks;  // never more splits than key blocks

@@ -542,6 +542,8 @@ int launch_fwd_d32(const FwdArgs& a, int variant, int nb, hipStream_t st);
 int launch_fwd_d64(const FwdArgs& a, int variant, int nb, hipStream_t st);
 int launch_fwd_d96(const FwdArgs& a, int variant, int nb, hipStream_t st);
 int launch_fwd_d128(const FwdArgs& a, int variant, int nb, hipStream_t st);
+// whether launch_fwd_d128 takes the 8-wave kernel (256 query rows per work-group instead of 128)
+bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr);
 
 template <int D, int NB, int VAR>
 inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
