@@ -351,7 +351,8 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                 }
             l_run[nb] += rs;  // per-lane partial; the two half-waves are added in the epilogue
             if constexpr (kDropout) {
-                // drop iff word < threshold, survivors * 1/(1-p), row sum left undropped (src/flash_forward.h:221-237)
+                // drop iff field < threshold, row sum left undropped (src/flash_forward.h:221-237); the survivors' factor
+                // 1/(1-p) is common to the whole row and multiplies O once in the epilogue instead of every score here
                 const uint32_t i_u = (uint32_t)row_i[nb];
                 uint8_t* kout = a.keep_out ? a.keep_out + ((size_t)bh * Nq + row_i[nb]) * Nk : nullptr;
 #pragma unroll
@@ -364,7 +365,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
 #pragma unroll
                         for (int f = 0; f < 8; ++f) {
                             const int r = 8 * q + f;
-                            s[kb][nb][r] = philox_field16(w, f) >= a.drop_thr ? s[kb][nb][r] * a.drop_rscale : 0.0f;
+                            s[kb][nb][r] = philox_field16(w, f) >= a.drop_thr ? s[kb][nb][r] : 0.0f;
                         }
                         if (a.keep_out != nullptr) {  // debug dump: one uniform branch per call, none per score
 #pragma unroll
@@ -457,7 +458,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         const float l = xhalf_sum(l_run[nb]);
-        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+        const float inv = l > 0.0f ? (kDropout ? a.drop_rscale : 1.0f) / l : 0.0f;
         const float lse = l > 0.0f ? (m_ref[nb] + fast_log2(l)) * kLn2 : -INFINITY;
         const int i = row_i[nb];
         if (i >= Nq) continue;
@@ -511,7 +512,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
                 const float l = xhalf_sum(l_run[nb]);
-                const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+                const float inv = l > 0.0f ? (kDropout ? a.drop_rscale : 1.0f) / l : 0.0f;
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll

@@ -410,7 +410,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
 #pragma unroll
                     for (int f = 0; f < 8; ++f) {
                         const int r = 8 * q + f;
-                        s[kb][r] = philox_field16(w, f) >= a.drop_thr ? s[kb][r] * a.drop_rscale : 0.0f;
+                        s[kb][r] = philox_field16(w, f) >= a.drop_thr ? s[kb][r] : 0.0f;  // the 1/(1-p) waits for the epilogue
                     }
                     if (a.keep_out != nullptr) {  // debug dump: one uniform branch per call, none per score
 #pragma unroll
@@ -521,7 +521,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     // ---------------- epilogue
     {
         const float l = xhalf_sum(l_run);
-        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+        const float inv = l > 0.0f ? (kDropout ? a.drop_rscale : 1.0f) / l : 0.0f;
         const float lse = l > 0.0f ? (m_ref + fast_log2(l)) * kLn2 : -INFINITY;
         if (a.num_splits > 1) {
             if (row_i < Nq) {
