@@ -41,6 +41,8 @@ enum {
  *   O (float*)                 O                fp16 [B,H,Nq,d]  (the reference stores fp32)
  *   --                         LSE              fp32 [B,H,Nq]    natural-log sum-exp of the masked scaled scores
  *   O_tmp, L, M                O_partial, LSE_partial   fp32 [B,H,S,Nq,d] and [B,H,S,Nq]; LSE_s = M_s + log L_s
+ *                                               (scratch of one call: with Nq == 1 and four or more query heads per
+ *                                               K/V head the order inside is [B,H_kv,S,H/H_kv,d] and [B,H_kv,S,H/H_kv])
  *   N, d (+ gridDim.y/.z)      B, H, Nq, Nk, d
  *   Br,Bc,Tr,Tc                not part of the ABI (tiling is the library's business)
  *   softmax_scale              softmax_scale
