@@ -24,7 +24,6 @@
 //    element-wise load / store path (kVec = false).
 #pragma once
 #include "common.h"
-#include <cstdlib>
 
 namespace fa {
 
@@ -554,9 +553,7 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
     static bool attr_done[kMaxDevices] = {};  // per instantiation and device
     if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), C::SMEM, attr_done); e != hipSuccess) return e;
     const long long groups = (long long)a.Tr * a.B * a.H * a.num_splits;
-    static const int pad = getenv("FA_LDS_PAD") ? atoi(getenv("FA_LDS_PAD")) : 0;
-    if (pad) hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM + pad);
-    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(256), C::SMEM + pad, st, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(256), C::SMEM, st, a);
     return hipGetLastError();
 }
 
