@@ -72,40 +72,50 @@ def test_graph_capture_and_replay(fa, mode):
 
 
 def test_random_shape_sweep(fa, oracle):
-    """32 seeded random problems: sizes around the tile edges, every mask family, ALiBi, grouped K/V heads, with and
-    without key splits."""
+    """200 seeded random problems: sizes around the tile edges and beyond the 8-wave kernel's thresholds, every mask
+    family, ALiBi, non-default scales, dropout, grouped K/V heads, with explicit, automatic and no key splits."""
     import torch
 
     rng = np.random.default_rng(2024)
-    dims = [8, 16, 31, 32, 40, 64, 72, 96, 100, 128]
-    for case in range(32):
+    dims = [8, 16, 31, 32, 40, 64, 64, 72, 96, 100, 128, 128, 128]
+    for case in range(200):
         d = int(rng.choice(dims))
-        B, Hk = int(rng.integers(1, 3)), int(rng.integers(1, 4))
-        H = Hk * int(rng.choice([1, 1, 2, 4]))
-        Nq = int(rng.choice([1, 7, 64, 65, 129, 200, 257, 300]))
-        Nk = Nq if rng.random() < 0.5 else int(rng.integers(1, 700))
+        B, Hk = int(rng.integers(1, 3)), int(rng.integers(1, 3))
+        H = Hk * int(rng.choice([1, 1, 2, 4, 8]))
+        Nq = int(rng.choice([1, 1, 7, 64, 65, 129, 200, 257, 300, 511, 640, 1025, 1100, 1400]))
+        Nk = Nq if rng.random() < 0.5 else int(rng.integers(1, 1600))
         fam = int(rng.integers(0, 4))
         kw, okw = {}, {}
         if fam == 1:
             kw = okw = dict(causal=True)
         elif fam == 2:
-            w = (int(rng.integers(0, 300)), int(rng.integers(0, 300)))
+            w = (int(rng.integers(0, 700)), int(rng.integers(0, 700)))
             kw, okw = dict(window=w), dict(window=w)
         elif fam == 3:
-            w = (int(rng.integers(0, 200)), -1)
+            w = (int(rng.integers(0, 800)), -1)
             kw, okw = dict(causal=True, window=w), dict(causal=True, window=w)
         if rng.random() < 0.3:
             sl = oracle.alibi_slopes(H)
             kw = dict(kw, alibi_slopes=torch.from_numpy(sl).cuda())
             okw = dict(okw, slopes=sl)
+        if rng.random() < 0.15:
+            sc = float(rng.choice([0.02, 0.3, -0.1]))
+            kw, okw = dict(kw, softmax_scale=sc), dict(okw, scale=sc)
         q = randn_f16_gpu((B, H, Nq, d), 1000 + case)
         k = randn_f16_gpu((B, Hk, Nk, d), 2000 + case)
         v = randn_f16_gpu((B, Hk, Nk, d), 3000 + case)
         kr, vr = (t.repeat_interleave(H // Hk, dim=1).contiguous() for t in (k, v))
-        O, L = oracle_forward_batched(oracle, q, kr, vr, **okw)
         what = f"case {case}: B{B} H{H}/{Hk} Nq{Nq} Nk{Nk} d{d} {sorted(kw)}"
+        S = int(rng.integers(0, 6))  # 0: the library chooses
+        if rng.random() < 0.25:
+            p = float(rng.choice([0.1, 0.5, 0.77]))
+            seed, off = int(rng.integers(0, 2 ** 40)), int(rng.integers(0, 2 ** 33))
+            keep = oracle.dropout_keep_mask(seed, off, p, B, H, Nq, Nk)
+            okw = dict(okw, keep_mask=torch.from_numpy(keep), p_drop=p)
+            kw = dict(kw, dropout_p=p, seed=seed, offset=off)
+            what += f" dropout {p}"
+        O, L = oracle_forward_batched(oracle, q, kr, vr, **okw)
         o, lse = fa.flash_forward(q, k, v, **kw)
         check_o_lse(o, lse, O, L, what)
-        S = int(rng.integers(2, 6))
         o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=S, **kw)
         check_o_lse(o, lse, O, L, what + f" split {S}")
