@@ -38,6 +38,7 @@ class FlashParams(C.Structure):
         ("num_splits", C.c_int),
         ("keep_mask_out", C.c_void_p),
         ("H_kv", C.c_int),
+        ("scores_out", C.c_void_p),
     ]
 
 
@@ -81,6 +82,10 @@ def lib():
         L.flash_last_hip_error.restype = C.c_char_p
         L.flash_strerror.restype = C.c_char_p
         L.flash_strerror.argtypes = [C.c_int]
+        L.flash_params_size.restype = C.c_size_t
+        if L.flash_params_size() != C.sizeof(FlashParams):
+            raise ImportError(f"{_LIB_PATH} was built with another flash_params ({L.flash_params_size()} bytes, this "
+                              f"binding: {C.sizeof(FlashParams)}): rebuild the library")
         _lib = L
     return _lib
 
@@ -112,7 +117,8 @@ def _check_qkv(q, k, v):
 
 
 def make_params(q, k, v, o, lse, softmax_scale=None, causal=False, window=(-1, -1), alibi_slopes=None,
-                dropout_p=0.0, seed=0, offset=0, num_splits=1, o_partial=None, lse_partial=None, keep_mask_out=None):
+                dropout_p=0.0, seed=0, offset=0, num_splits=1, o_partial=None, lse_partial=None, keep_mask_out=None,
+                scores_out=None):
     B, H, Nq, Nk, d = _check_qkv(q, k, v)
     p = FlashParams()
     p.Q, p.K, p.V, p.O, p.LSE = _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse)
@@ -127,14 +133,16 @@ def make_params(q, k, v, o, lse, softmax_scale=None, causal=False, window=(-1, -
     p.num_splits = int(num_splits)
     p.keep_mask_out = _ptr(keep_mask_out)
     p.H_kv = int(k.shape[1])
+    p.scores_out = _ptr(scores_out)
     return p
 
 
 def flash_forward(q, k, v, softmax_scale=None, causal=False, window=(-1, -1), alibi_slopes=None, dropout_p=0.0,
-                  seed=0, offset=0, return_keep_mask=False, stream=None, out=None, lse=None):
+                  seed=0, offset=0, return_keep_mask=False, stream=None, out=None, lse=None, scores_out=None):
     """O = softmax(mask(Q K^T * scale - slope * |i - j|)) V over the whole key range.
     q [B,H,Nq,d], k,v [B,H,Nk,d] fp16 on the GPU.  Returns (O fp16 [B,H,Nq,d], LSE fp32 [B,H,Nq]) and, when
-    return_keep_mask, the uint8 keep decisions [B,H,Nq,Nk] the kernel applied."""
+    return_keep_mask, the uint8 keep decisions [B,H,Nq,Nk] the kernel applied.  scores_out: optional fp32
+    [B,H,Nq,Nk] tensor (pre-filled with -inf) that receives the visible scores (debug; slow kernel instance)."""
     import torch
 
     B, H, Nq, Nk, d = _check_qkv(q, k, v)
@@ -142,7 +150,7 @@ def flash_forward(q, k, v, softmax_scale=None, causal=False, window=(-1, -1), al
     l = lse if lse is not None else torch.empty((B, H, Nq), dtype=torch.float32, device=q.device)
     km = torch.zeros((B, H, Nq, Nk), dtype=torch.uint8, device=q.device) if return_keep_mask else None
     p = make_params(q, k, v, o, l, softmax_scale, causal, window, alibi_slopes, dropout_p, seed, offset, 1,
-                    keep_mask_out=km)
+                    keep_mask_out=km, scores_out=scores_out)
     rc = lib().flash_forward(C.byref(p), _stream_handle(stream))
     if rc != FLASH_OK:
         raise FlashError(rc, "flash_forward")
@@ -151,7 +159,7 @@ def flash_forward(q, k, v, softmax_scale=None, causal=False, window=(-1, -1), al
 
 def flash_forward_splitkv(q, k, v, num_splits=0, softmax_scale=None, causal=False, window=(-1, -1),
                           alibi_slopes=None, dropout_p=0.0, seed=0, offset=0, stream=None, workspace=None,
-                          return_partials=False, out=None, lse=None):
+                          return_partials=False, out=None, lse=None, scores_out=None):
     """Split-KV forward + combine.  num_splits <= 0 asks the library's heuristic.  `workspace` may carry a
     pre-allocated (O_partial, LSE_partial) pair; otherwise it is allocated here (the caller owns the workspace, as
     in src/main.cu:160-162)."""
@@ -160,7 +168,8 @@ def flash_forward_splitkv(q, k, v, num_splits=0, softmax_scale=None, causal=Fals
     B, H, Nq, Nk, d = _check_qkv(q, k, v)
     o = out if out is not None else torch.empty((B, H, Nq, d), dtype=torch.float16, device=q.device)
     l = lse if lse is not None else torch.empty((B, H, Nq), dtype=torch.float32, device=q.device)
-    p = make_params(q, k, v, o, l, softmax_scale, causal, window, alibi_slopes, dropout_p, seed, offset, num_splits)
+    p = make_params(q, k, v, o, l, softmax_scale, causal, window, alibi_slopes, dropout_p, seed, offset, num_splits,
+                    scores_out=scores_out)
     if workspace is None:
         ob, lb = C.c_size_t(), C.c_size_t()
         rc = lib().flash_splitkv_workspace_bytes(C.byref(p), C.byref(ob), C.byref(lb))

@@ -34,6 +34,7 @@ struct FwdArgs {
     float* LSE_partial;  // [B,H,S,Nq]   fp32, m_s + log l_s   (reference M, L)
     const float* alibi;  // [H] or nullptr
     uint8_t* keep_out;   // [B,H,Nq,Nk] or nullptr
+    float* scores_out;   // [B,H,Nq,Nk] or nullptr (element-wise instance of the 4-wave kernel only)
     int B, H, Nq, Nk, d;
     int Hk, kv_group;    // K/V heads and query heads per K/V head (H = Hk * kv_group)
     int causal, wl, wr;  // wl / wr < 0: unbounded

@@ -56,6 +56,7 @@ int validate(const flash_params* p, bool* empty)
     if (misaligned(p->Q, need) || misaligned(p->O, need) || misaligned(p->LSE, 4)) return FLASH_EALIGN;
     if (p->Nk > 0 && (misaligned(p->K, need) || misaligned(p->V, need))) return FLASH_EALIGN;
     if (p->alibi_slopes && misaligned(p->alibi_slopes, 4)) return FLASH_EALIGN;
+    if (p->scores_out && misaligned(p->scores_out, 4)) return FLASH_EALIGN;
     return FLASH_OK;
 }
 
@@ -73,6 +74,7 @@ void fill_args(const flash_params* p, int splits, fa::FwdArgs* a)
     a->LSE_partial = p->LSE_partial;
     a->alibi = p->alibi_slopes;
     a->keep_out = p->dropout_p > 0.0f ? p->keep_mask_out : nullptr;
+    a->scores_out = p->scores_out;
     a->B = p->B;
     a->H = p->H;
     a->Nq = p->Nq;
@@ -98,7 +100,7 @@ void fill_args(const flash_params* p, int splits, fa::FwdArgs* a)
 int launch_tiled(const flash_params* p, const fa::FwdArgs& a, hipStream_t st)
 {
     // A non-positive scale does not commute with the row maximum: only the element-wise instance scales first.
-    int variant = (p->d % 8 == 0 && p->softmax_scale > 0.0f) ? 1 : 0;
+    int variant = (p->d % 8 == 0 && p->softmax_scale > 0.0f && !p->scores_out) ? 1 : 0;  // (the score dump lives there too)
     if (p->alibi_slopes) variant |= 2;
     if (p->dropout_p > 0.0f) variant |= 4;
     int e;
@@ -169,7 +171,9 @@ FLASH_EXPORT int flash_forward_splitkv(const flash_params* p, void* stream)
     fa::FwdArgs a;
     fill_args(p, splits, &a);
     int e;
-    if (p->Nq == 1 && a.kv_group >= 4 && !p->alibi_slopes && p->window_left < 0 && p->dropout_p == 0.0f) {
+    if (p->scores_out) {
+        e = launch_tiled(p, a, st);  // debug dump: element-wise instance of the tiled kernel
+    } else if (p->Nq == 1 && a.kv_group >= 4 && !p->alibi_slopes && p->window_left < 0 && p->dropout_p == 0.0f) {
         // Decode with grouped K/V heads: the G query heads of one K/V head, one row each, are the G rows of one
         // attention problem over that K/V head -- Q [B,H,1,d] is [B,H_kv,G,d] in memory, and so are O, LSE and the
         // split workspace, and no mask depends on the row.  The tiled kernel then streams K/V once per K/V head and
@@ -253,6 +257,8 @@ FLASH_EXPORT int flash_dropout_keep_mask(const flash_params* p, uint8_t* mask_ou
     return record_hip(fa::launch_keep_mask(mask_out, p->B, p->H, p->Nq, p->Nk, flash_dropout_threshold(p->dropout_p),
                                            p->seed, p->offset, static_cast<hipStream_t>(stream)));
 }
+
+FLASH_EXPORT size_t flash_params_size(void) { return sizeof(flash_params); }
 
 FLASH_EXPORT const char* flash_last_hip_error(void) { return g_hip_error; }
 

@@ -320,6 +320,19 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                         }
                 }
             }
+            if constexpr (!kVec) {
+                if (a.scores_out != nullptr && row_i[nb] < Nq) {  // debug dump of the visible scores, natural-log units
+                    float* srow = a.scores_out + ((size_t)bh * Nq + row_i[nb]) * Nk;
+                    const float unit = (scale_late ? cs : 1.0f) * kLn2;
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const int j = kb0 + 4 * g + 32 * kb + 8 * (r >> 2) + (r & 3);
+                            if (j >= lo[nb] && j <= hi[nb]) srow[j] = s[kb][nb][r] * unit;
+                        }
+                }
+            }
             float mx = -INFINITY;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)

@@ -80,6 +80,12 @@ typedef struct flash_params {
      * K/V head h / (H / H_kv).  0 means H (one K/V head per query head, all the reference can express: it indexes
      * K and V with the query head, src/flash_forward.h:57-59).  H must be a multiple of H_kv. */
     int H_kv;
+    /* Optional debug output: when non-NULL, the forward also stores the scores the softmax is taken over,
+     * softmax_scale * q_i.k_j - slope_h * |i - j| in fp32, for every (i, j) that the masks leave visible, into
+     * scores_out [B,H,Nq,Nk]; entries of masked pairs are not written (fill the buffer with -inf beforehand to read it
+     * as the masked score matrix).  The call then takes the element-wise kernel instance, which serves every
+     * feature but is several times slower.  No counterpart in the reference. */
+    float *scores_out;
 } flash_params;
 
 /* Tiled forward over the whole key range: replaces
@@ -118,6 +124,10 @@ int flash_dropout_keep_mask(const flash_params *p, uint8_t *mask_out, void *stre
  * up of output word f >> 1), and element (i, j) is kept iff field 4*((j >> 3) & 1) + (j & 3) >= threshold.  Kept
  * probabilities are scaled by 1/(1 - dropout_p); the row sum of the softmax is taken before the drop. */
 uint32_t flash_dropout_threshold(float dropout_p);
+
+/* sizeof(flash_params) of the header the library was built with.  A caller compiled against another version of the
+ * header would hand over a struct of another size (fields are only ever appended): compare before the first call. */
+size_t flash_params_size(void);
 
 /* Text of the last HIP error seen by this thread inside the library ("" if none). */
 const char *flash_last_hip_error(void);

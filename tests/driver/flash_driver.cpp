@@ -178,6 +178,11 @@ int main(int argc, char** argv)
     HIP_CHECK(hipMemcpy(Kd, Kh.data(), n * 2, hipMemcpyHostToDevice));
     HIP_CHECK(hipMemcpy(Vd, Vh.data(), n * 2, hipMemcpyHostToDevice));
 
+    if (flash_params_size() != sizeof(flash_params)) {
+        std::fprintf(stderr, "libflash_attn_mi355.so was built with another flash_params (%zu bytes, this program: %zu): rebuild\n",
+                     flash_params_size(), sizeof(flash_params));
+        return 2;
+    }
     flash_params p;
     std::memset(&p, 0, sizeof(p));
     p.Q = Qd;

@@ -300,3 +300,51 @@ def test_eight_wave_kernel_cases(fa, oracle, Nq, Nk, Hk, kw):
     if p == 0.0:
         o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=3, **kw)
         check_o_lse(o, lse, O, L, f"8-wave split Nq={Nq} Nk={Nk} {sorted(kw)}")
+
+
+@pytest.mark.parametrize("Nq,Nk,d,Hk,kw", [
+    (200, 200, 64, 2, dict(causal=True)),
+    (130, 333, 128, 1, dict(window=(50, 20), alibi=True)),
+    (1, 700, 128, 1, dict()),                                  # decode with 8 query heads per K/V head
+    (300, 300, 31, 2, dict(causal=True, window=(100, -1), softmax_scale=-0.2)),
+])
+def test_score_dump(fa, oracle, Nq, Nk, d, Hk, kw):
+    """The optional score matrix is the one the result was computed from: its -inf pattern is the mask, its row-wise
+    log-sum-exp is the LSE output, and softmax(scores) V is O -- for the plain and for the split entry point."""
+    import torch
+    B, H = 2, 8 if Nq == 1 else 2
+    q = randn_f16_gpu((B, H, Nq, d), 31)
+    k = randn_f16_gpu((B, Hk, Nk, d), 32)
+    v = randn_f16_gpu((B, Hk, Nk, d), 33)
+    kw = dict(kw)
+    okw = {x: kw[x] for x in ("causal", "window") if x in kw}
+    if "softmax_scale" in kw:
+        okw["scale"] = kw["softmax_scale"]
+    if kw.pop("alibi", False):
+        sl, sl_t = _slopes(oracle, H)
+        kw["alibi_slopes"], okw["slopes"] = sl_t, sl
+    kr, vr = (t.repeat_interleave(H // Hk, dim=1).contiguous() for t in (k, v))
+    O, L = oracle_forward_batched(oracle, q, kr, vr, **okw)
+    ii = np.arange(Nq)[:, None] + (Nk - Nq)
+    jj = np.arange(Nk)[None, :]
+    wl, wr = kw.get("window", (-1, -1))
+    vis = np.ones((Nq, Nk), dtype=bool)
+    if kw.get("causal"):
+        vis &= jj <= ii
+    if wl >= 0:
+        vis &= jj >= ii - wl
+    if wr >= 0:
+        vis &= jj <= ii + wr
+    for entry, extra in ((fa.flash_forward, {}), (fa.flash_forward_splitkv, dict(num_splits=3))):
+        sc = torch.full((B, H, Nq, Nk), float("-inf"), dtype=torch.float32, device="cuda")
+        o, lse = entry(q, k, v, scores_out=sc, **extra, **kw)
+        check_o_lse(o, lse, O, L, f"score dump {entry.__name__}")
+        S = sc.cpu().numpy().astype(np.float64)
+        assert np.array_equal(np.isfinite(S), np.broadcast_to(vis, S.shape)), "-inf pattern is not the mask"
+        m = np.where(vis.any(1), np.max(np.where(vis, S, -np.inf), axis=-1), 0.0)
+        P = np.where(vis, np.exp(S - m[..., None]), 0.0)
+        l = P.sum(-1)
+        rows = vis.any(1)
+        assert np.abs((m + np.log(np.where(l > 0, l, 1.0)))[..., rows] - L[..., rows]).max() <= 1e-4
+        Oref = np.einsum("bhij,bhjd->bhid", P / np.where(l > 0, l, 1.0)[..., None], to_f32_np(vr).astype(np.float64))
+        assert np.abs(Oref - O).max() <= 2e-3
