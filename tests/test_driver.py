@@ -28,6 +28,13 @@ def test_driver_is_built_and_prints_usage():
     assert _run("--seq", "0").returncode == 2
 
 
+def test_driver_is_not_older_than_the_header():
+    """A driver built against an older flash_params would hand the library a short struct; `make -q` says whether the
+    binary is up to date with flash_driver.cpp and the public header.  (The binary also checks flash_params_size().)"""
+    r = subprocess.run(["make", "-q", "-C", os.path.join(ROOT, "tests", "driver"), "flash_driver"], capture_output=True)
+    assert r.returncode == 0, "tests/driver/flash_driver is stale: run `make -C tests/driver`"
+
+
 def test_mfma_rate_probe_is_built():
     assert os.path.exists(os.path.join(ROOT, "tests", "driver", "mfma_rate")), "run `make -C tests/driver`"
 
