@@ -107,6 +107,19 @@ __device__ __forceinline__ v4u philox4x32_10(uint32_t c0, uint32_t c1, uint32_t 
 // 16-bit field f (0..7) of a Philox output
 __device__ __forceinline__ uint32_t philox_field16(const v4u& w, int f) { return (w[f >> 1] >> (16 * (f & 1))) & 0xffffu; }
 
+// One KiB from global memory straight into LDS: lane l fetches 16 bytes at base + off (its own offset) and the wave
+// writes them to lds_dst + 16 l.  Issued as inline asm on purpose: the compiler models the builtin form as a FLAT
+// access that may touch LDS, and from then on degrades every LDS wait of the loop to "wait for everything".  The
+// caller waits with s_waitcnt vmcnt(0) before the barrier that publishes the tile.
+__device__ __forceinline__ void dma_kib(const char* base, uint32_t off, FA_LDS char* lds_dst)
+{
+    const uint32_t m0v = (uint32_t)(uintptr_t)lds_dst;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(m0v), "v"(off), "s"(base)
+                 : "memory", "m0");
+}
+
 // Raises the dynamic-LDS limit of a kernel once per device (the attribute belongs to the device's copy of the kernel).
 // `done` is the caller's per-kernel flag array; concurrent first calls may both set the attribute, which is harmless.
 constexpr int kMaxDevices = 64;

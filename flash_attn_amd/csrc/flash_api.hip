@@ -131,7 +131,7 @@ int resolve_splits(const flash_params* p)
         s = (int)(want < by_keys ? want : by_keys);
     } else if (s <= 0) {
         const bool vec = p->d % 8 == 0 && p->softmax_scale > 0.0f;
-        const int rows = fa::fwd_uses_pingpong(p->d, vec, p->Nq, p->is_causal, p->window_left, p->window_right) ? 256 : kRowsPerGroup;
+        const int rows = fa::fwd_uses_pingpong(p->d, vec, p->Nq, p->is_causal, p->window_left, p->window_right, (long long)p->B * p->H) ? 256 : kRowsPerGroup;
         const int Tr = (p->Nq + rows - 1) / rows;
         // argument roles as in the reference's call (src/main.cu:125), with the CU count of the MI355X and the row
         // blocks of the kernel that will run

@@ -27,6 +27,10 @@
 
 namespace fa {
 
+#ifndef FA_DMA_MIN_D
+#define FA_DMA_MIN_D 128
+#endif
+
 template <int D, int NB>
 struct FwdCfg {
     static constexpr int kWaves = 4;
@@ -47,6 +51,13 @@ struct FwdCfg {
     static constexpr int KBUF = BC * SK;
     static constexpr int VBUF = BC * SV;
     static constexpr int SMEM = 2 * KBUF + 2 * VBUF;
+    // At D >= FA_DMA_MIN_D the instances whose rows are whole 16-byte chunks of exactly D columns fetch their tiles
+    // straight into LDS (global_load_lds_dwordx4) instead of through registers.
+    static constexpr bool DMA = D >= FA_DMA_MIN_D;
+    static constexpr int NSTG = 2;
+    static constexpr int SMEM_DMA = NSTG * (KBUF + VBUF);
+    static constexpr int NKX = (CH + 1 + 3) / 4;  // 1 KiB blocks of a K tile (CH + 1 of them) per wave, rounded up
+    static constexpr int NVX = CH / 4;            // 1 KiB blocks of a V tile (CH of them) per wave
     static constexpr int NLD = BC * CH / 256;  // 16-byte chunks per thread per tile (K and V each)
     static_assert(D % 32 == 0 && D <= 128, "head-dim bucket");
     static_assert((BC * CH) % 256 == 0, "tile chunks must divide over the group");
@@ -91,9 +102,11 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                    kFullD = (VAR & kVarFullD) != 0;
     using C = FwdCfg<D, NB>;
     constexpr int BC = C::BC, KS = C::KS, MB = C::MB, CH = C::CH, SK = C::SK, SV = C::SV, NLD = C::NLD;
+    constexpr bool kDma = C::DMA && kVec && kFullD;
+    constexpr int NSTG = kDma ? C::NSTG : 2;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     char* const Ks = smem;
-    char* const Vs = smem + 2 * C::KBUF;
+    char* const Vs = smem + NSTG * C::KBUF;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -215,6 +228,57 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
         for (int x = 0; x < NLD; ++x)
             *reinterpret_cast<v4u*>(Vs + buf * C::VBUF + ld_row[x] * SV +
                                     ((ld_col[x] * 2) ^ (C::VSWZ ? ((ld_row[x] >> 1) & 1) << 6 : 0))) = vreg[x];
+    };
+
+    // ---- direct global -> LDS path: the tile buffers keep their layout (K rows padded by one chunk, V rows with the
+    // 64-byte halves exchanged in rows 2, 3 mod 4), and a request fills 64 consecutive 16-byte chunks of a buffer: lane l of
+    // block x fetches whatever belongs into chunk 64 x + l (the pad chunk of a K row gets a copy of its neighbour).
+    // Blocks go round the four waves; the odd K block goes to the waves that still have a block index left for it.
+    uint32_t koff[C::NKX], voff[C::NVX];
+    int krow[C::NKX], vrow[C::NVX];
+    if constexpr (kDma) {
+#pragma unroll
+        for (int i = 0; i < C::NKX; ++i) {
+            const int q = 64 * (wave + 4 * i) + lane;
+            krow[i] = q / (CH + 1);
+            const int col = q % (CH + 1);
+            koff[i] = (uint32_t)(krow[i] * D * 2 + (col < CH ? col : CH - 1) * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < C::NVX; ++i) {
+            const int q = 64 * (wave + 4 * i) + lane;
+            vrow[i] = q / CH;
+            const int c = q % CH;
+            voff[i] = (uint32_t)(vrow[i] * D * 2 + (C::VSWZ ? c ^ (((vrow[i] >> 1) & 1) << 2) : c) * 16);
+        }
+    }
+    const bool k_extra = wave + 4 * (C::NKX - 1) <= CH;  // the last round of K blocks exists for this wave
+    auto dma_tile = [&](int tile, int stage) {
+        const uint32_t tb = (uint32_t)tile * (uint32_t)(BC * D * 2);
+        const int rows_left = Nk - tile * BC;  // >= 1; keys past Nk re-read key Nk - 1 (their scores are masked)
+        FA_LDS char* const kst = (FA_LDS char*)smem + stage * C::KBUF;
+        FA_LDS char* const vst = (FA_LDS char*)smem + NSTG * C::KBUF + stage * C::VBUF;
+        const char* const Kb = reinterpret_cast<const char*>(Kbh);
+        const char* const Vb = reinterpret_cast<const char*>(Vbh);
+#pragma unroll
+        for (int i = 0; i < C::NKX; ++i) {
+            if (i == C::NKX - 1 && !k_extra) break;
+            uint32_t o = koff[i] + tb;
+            if (rows_left < BC && krow[i] >= rows_left) o -= (uint32_t)((krow[i] - rows_left + 1) * D * 2);
+            dma_kib(Kb, o, kst + (wave + 4 * i) * 1024);
+        }
+#pragma unroll
+        for (int i = 0; i < C::NVX; ++i) {
+            uint32_t o = voff[i] + tb;
+            if (rows_left < BC && vrow[i] >= rows_left) o -= (uint32_t)((vrow[i] - rows_left + 1) * D * 2);
+            dma_kib(Vb, o, vst + (wave + 4 * i) * 1024);
+        }
+    };
+    // wait until at most the requests of one tile (the youngest) are still in flight / until none is
+    auto dma_wait = [&](bool one_tile_in_flight) {
+        if (!one_tile_in_flight) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        else if (k_extra) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(C::NKX + C::NVX) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(C::NKX + C::NVX - 1) : "memory");
     };
 
     // ---- accumulators
@@ -430,40 +494,68 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
             for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[nb][ks]));
     };
 
-    // ---- double-buffered loop: tile t+1 is fetched from global memory while tile t is computed
-    if (ntiles > 0) {
-        gload(Kbh, tile_begin, kreg);
-        gload(Vbh, tile_begin, vreg);
-        put_k(0);
-        put_v(0);
-    }
-    pin_q();
-    __syncthreads();
+    // ---- loop over the key tiles
     // A wave whose rows all lie past Nq (fewer than 128 query rows: short prompts, or the heads of one K/V head decoding
     // together) only helps to stage the tiles, and so does any wave for a tile that none of its rows can see (the far
     // end of the causal diagonal block, the near end of a sliding window).
     const bool wave_live = q0 + wave * C::RW < Nq;
-    for (int t = 0; t < ntiles; ++t) {
-        const int cur = t & 1;
+    auto tile_math = [&](int t, int buf) {
         const int kb0 = (tile_begin + t) * BC;
-        const bool has1 = t + 1 < ntiles;
-        if (has1) {
-            gload(Kbh, tile_begin + t + 1, kreg);
-            gload(Vbh, tile_begin + t + 1, vreg);
-        }
         if (wave_live && kb0 <= hi_max && kb0 + BC - 1 >= lo_min) {
             v16f s[2][NB];
             v8h pf[2][2][NB];
-            qk(cur, s);
+            qk(buf, s);
             const int mask_sides = (kb0 < lo_max ? 1 : 0) | (kb0 + BC - 1 > hi_min ? 2 : 0);
             softmax(mask_sides, kb0, s, pf);
-            pv(cur, pf);
+            pv(buf, pf);
         }
-        if (has1) {
-            put_k(cur ^ 1);
-            put_v(cur ^ 1);
-        }
+    };
+    if constexpr (kDma) {
+        // Tile t + PF is requested when tile t starts (its stage was read last during tile t - 1, behind a barrier);
+        // before the barrier that ends tile t, the requests of tile t + 1 have landed, those of t + 2 may be in flight.
+        constexpr int PF = NSTG - 1;
+        static_assert(PF == 1 || PF == 2, "prefetch distance");
+        static_assert(C::NKX + C::NVX <= 15, "vmcnt immediate");
+#pragma unroll
+        for (int u = 0; u < PF; ++u)
+            if (u < ntiles) dma_tile(tile_begin + u, u);
+        dma_wait(PF == 2 && ntiles > 1);
+        pin_q();
         __syncthreads();
+        int buf = 0, nbuf = PF % NSTG;  // stages of tile t and of tile t + PF
+        for (int t = 0; t < ntiles; ++t) {
+            const bool more = t + PF < ntiles;
+            if (more) dma_tile(tile_begin + t + PF, nbuf);
+            tile_math(t, buf);
+            dma_wait(PF == 2 && more);
+            __syncthreads();
+            buf = buf + 1 == NSTG ? 0 : buf + 1;
+            nbuf = nbuf + 1 == NSTG ? 0 : nbuf + 1;
+        }
+    } else {
+        // double-buffered through registers: tile t+1 is fetched from global memory while tile t is computed
+        if (ntiles > 0) {
+            gload(Kbh, tile_begin, kreg);
+            gload(Vbh, tile_begin, vreg);
+            put_k(0);
+            put_v(0);
+        }
+        pin_q();
+        __syncthreads();
+        for (int t = 0; t < ntiles; ++t) {
+            const int cur = t & 1;
+            const bool has1 = t + 1 < ntiles;
+            if (has1) {
+                gload(Kbh, tile_begin + t + 1, kreg);
+                gload(Vbh, tile_begin + t + 1, vreg);
+            }
+            tile_math(t, cur);
+            if (has1) {
+                put_k(cur ^ 1);
+                put_v(cur ^ 1);
+            }
+            __syncthreads();
+        }
     }
 
     // ---------------- epilogue: normalise once, store O (fp16) + LSE, or the fp32 split partials
@@ -556,7 +648,8 @@ int launch_fwd_d64(const FwdArgs& a, int variant, int nb, hipStream_t st);
 int launch_fwd_d96(const FwdArgs& a, int variant, int nb, hipStream_t st);
 int launch_fwd_d128(const FwdArgs& a, int variant, int nb, hipStream_t st);
 // whether launch_fwd_d128 takes the 8-wave kernel (256 query rows per work-group instead of 128)
-bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr);
+// (slices = B * H * num_splits)
+bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr, long long slices);
 
 template <int D, int NB, int VAR>
 inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
@@ -564,9 +657,10 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
     using C = FwdCfg<D, NB>;
     auto kern = fwd_kernel<D, NB, VAR>;
     static bool attr_done[kMaxDevices] = {};  // per instantiation and device
-    if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), C::SMEM, attr_done); e != hipSuccess) return e;
+    constexpr int smem = (C::DMA && (VAR & kVarVec) && (VAR & kVarFullD)) ? C::SMEM_DMA : C::SMEM;
+    if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, attr_done); e != hipSuccess) return e;
     const long long groups = (long long)a.Tr * a.B * a.H * a.num_splits;
-    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(256), C::SMEM, st, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(256), smem, st, a);
     return hipGetLastError();
 }
 

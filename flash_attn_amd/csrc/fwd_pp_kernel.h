@@ -41,19 +41,6 @@ struct PPCfg {
     static_assert(D == 64 || D == 128, "ping-pong kernel: head dim 64 or 128");
 };
 
-// One KiB from global memory straight into LDS: lane l fetches 16 bytes at base + off (its own offset) and the wave
-// writes them to lds_dst + 16 l.  Issued as inline asm on purpose: the compiler models the builtin form as a FLAT
-// access that may touch LDS, and from then on degrades every LDS wait of the loop to "wait for everything".  The
-// caller waits with s_waitcnt vmcnt(0) before the barrier that publishes the tile.
-__device__ __forceinline__ void dma_kib(const char* base, uint32_t off, FA_LDS char* lds_dst)
-{
-    const uint32_t m0v = (uint32_t)(uintptr_t)lds_dst;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(m0v), "v"(off), "s"(base)
-                 : "memory", "m0");
-}
-
 // LDS-only barrier: global loads in flight are not waited for.
 // The sched_barrier fences keep the compiler from moving ALU work of one phase across the barrier into the other.
 __device__ __forceinline__ void lds_barrier()

@@ -262,8 +262,8 @@ def test_full_size_properties_decode(fa):
     assert torch.allclose(o.float(), torch.full_like(o, 0.5, dtype=torch.float32), atol=1e-3)
 
 
-# The 8-wave kernel serves d = 128 with more than 1024 causal rows (or more than 128 rows without a causal mask):
-# ragged lengths beyond that threshold, Nq != Nk in both directions, every mask, grouped heads, dropout, split mode.
+# The 8-wave kernel (d = 128; by preference only large grids of long rows, forced here through FLASH_ATTN_KERNEL):
+# ragged lengths, Nq != Nk in both directions, every mask incl. narrow windows, grouped heads, dropout, split mode.
 @pytest.mark.parametrize("Nq,Nk,Hk,kw", [
     (1100, 1100, 2, dict(causal=True)),
     (1100, 1333, 2, dict(causal=True)),
@@ -273,9 +273,13 @@ def test_full_size_properties_decode(fa):
     (1100, 1100, 2, dict(causal=True, alibi=True)),
     (1061, 1061, 2, dict(causal=True, dropout_p=0.2, seed=99, offset=5)),
     (300, 1500, 2, dict(window=(700, 900))),
+    (300, 300, 2, dict(causal=True)),
+    (513, 700, 2, dict(window=(40, 3))),
+    (129, 129, 2, dict()),
 ])
-def test_eight_wave_kernel_cases(fa, oracle, Nq, Nk, Hk, kw):
+def test_eight_wave_kernel_cases(fa, oracle, Nq, Nk, Hk, kw, monkeypatch):
     import torch
+    monkeypatch.setenv("FLASH_ATTN_KERNEL", "8wave")
     B, H, d = 1, 2, 128
     q = randn_f16_gpu((B, H, Nq, d), 21)
     k = randn_f16_gpu((B, Hk, Nk, d), 22)
