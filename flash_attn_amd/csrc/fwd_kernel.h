@@ -331,6 +331,18 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                     s[kb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, qf[nb][ks], s[kb][nb], 0, 0, 0);
             }
         }
+        // issue order: kQkAhead fragment reads first, then read and MFMA in turn (left to itself the compiler waits
+        // for each fragment right after requesting it)
+        if constexpr (NB == 1) {
+            constexpr int kQkAhead = 3, n = 2 * KS;
+            __builtin_amdgcn_sched_group_barrier(0x100, kQkAhead, 0);
+#pragma unroll
+            for (int i = 0; i < n - kQkAhead; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, kQkAhead, 0);
+        }
     };
 
     // online softmax of one tile (per query row = per lane); leaves P^T packed to fp16 in pf
