@@ -27,9 +27,6 @@
 
 namespace fa {
 
-#ifndef FA_DMA_MIN_D
-#define FA_DMA_MIN_D 128
-#endif
 
 template <int D, int NB>
 struct FwdCfg {
@@ -51,9 +48,10 @@ struct FwdCfg {
     static constexpr int KBUF = BC * SK;
     static constexpr int VBUF = BC * SV;
     static constexpr int SMEM = 2 * KBUF + 2 * VBUF;
-    // At D >= FA_DMA_MIN_D the instances whose rows are whole 16-byte chunks of exactly D columns fetch their tiles
-    // straight into LDS (global_load_lds_dwordx4) instead of through registers.
-    static constexpr bool DMA = D >= FA_DMA_MIN_D;
+    // At D >= 96 the instances whose rows are whole 16-byte chunks of exactly D columns fetch their tiles straight into
+    // LDS (global_load_lds_dwordx4) instead of through registers (measured: +6-12 % at D = 128, +3-7 % at D = 96
+    // without dropout, -2.5 % with it, within +-2 % at D = 64).
+    static constexpr bool DMA = D >= 96;
     static constexpr int NSTG = 2;
     static constexpr int SMEM_DMA = NSTG * (KBUF + VBUF);
     static constexpr int NKX = (CH + 1 + 3) / 4;  // 1 KiB blocks of a K tile (CH + 1 of them) per wave, rounded up
@@ -102,7 +100,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                    kFullD = (VAR & kVarFullD) != 0;
     using C = FwdCfg<D, NB>;
     constexpr int BC = C::BC, KS = C::KS, MB = C::MB, CH = C::CH, SK = C::SK, SV = C::SV, NLD = C::NLD;
-    constexpr bool kDma = C::DMA && kVec && kFullD;
+    constexpr bool kDma = C::DMA && kVec && kFullD && (D >= 128 || !kDropout);
     constexpr int NSTG = kDma ? C::NSTG : 2;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     char* const Ks = smem;
@@ -669,7 +667,7 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
     using C = FwdCfg<D, NB>;
     auto kern = fwd_kernel<D, NB, VAR>;
     static bool attr_done[kMaxDevices] = {};  // per instantiation and device
-    constexpr int smem = (C::DMA && (VAR & kVarVec) && (VAR & kVarFullD)) ? C::SMEM_DMA : C::SMEM;
+    constexpr int smem = C::SMEM_DMA > C::SMEM ? C::SMEM_DMA : C::SMEM;  // (equal: both paths use two stages)
     if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, attr_done); e != hipSuccess) return e;
     const long long groups = (long long)a.Tr * a.B * a.H * a.num_splits;
     hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(256), smem, st, a);
