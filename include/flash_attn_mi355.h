@@ -61,7 +61,7 @@ typedef struct flash_params {
     float *LSE;
     float *O_partial;
     float *LSE_partial;
-    int B, H, Nq, Nk, d;
+    int B, H, Nq, Nk, d; /* one [N,d] slice of Q, K or V must stay below 4 GiB (N * d < 2^31) */
     float softmax_scale;
     int is_causal;
     int window_left;

@@ -84,6 +84,7 @@ def test_argument_errors_are_codes_not_aborts(fa):
         assert entry(C.byref(_params(fa, dropout_p=float("nan"))), None) == E_INVAL
         assert entry(C.byref(_params(fa, softmax_scale=float("inf"))), None) == E_INVAL
         assert entry(C.byref(_params(fa, num_splits=129)), None) == E_SPLITS
+        assert entry(C.byref(_params(fa, Nk=1 << 25, d=64)), None) == E_INVAL  # a K/V slice of 4 GiB
         assert entry(C.byref(_params(fa, H=6, H_kv=4)), None) == E_INVAL  # query heads must be a multiple of K/V heads
         assert entry(C.byref(_params(fa, H=2, H_kv=4)), None) == E_INVAL
         assert entry(C.byref(_params(fa, H=2, H_kv=-1)), None) == E_INVAL
