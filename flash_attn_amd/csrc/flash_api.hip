@@ -39,6 +39,8 @@ int validate_shape(const flash_params* p, bool* empty)
     if (!(p->dropout_p >= 0.0f && p->dropout_p < 1.0f)) return FLASH_EINVAL;
     if (p->num_splits > FLASH_MAX_SPLITS) return FLASH_ESPLITS;
     if ((long long)p->B * p->H > 0x7fffffffLL / 2) return FLASH_EINVAL;
+    // one-dimensional grids: slices x row blocks x splits must fit the 2^31 - 1 work-groups of a launch
+    if ((long long)p->B * p->H * ((p->Nq + 127) / 128) > 0x7fffffffLL / FLASH_MAX_SPLITS) return FLASH_EINVAL;
     // the tile requests address a [N,d] slice with 32-bit byte offsets
     if (2LL * p->Nq * p->d >= (1LL << 32) || 2LL * p->Nk * p->d >= (1LL << 32)) return FLASH_EINVAL;
     if (p->H_kv < 0 || (p->H_kv > 0 && (p->H_kv > p->H || p->H % p->H_kv != 0))) return FLASH_EINVAL;
