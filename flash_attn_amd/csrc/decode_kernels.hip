@@ -170,7 +170,7 @@ __global__ void __launch_bounds__(256) decode_split_kernel(const FwdArgs a)
                 o += w * s_acc[gI][tid];
             }
             const float inv = L > 0.0f ? 1.0f / L : 0.0f;
-            const float lse = L > 0.0f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
+            const float lse = L > 0.0f ? __builtin_fmaf(M, kLn2, fast_log2(L) * kLn2) : -INFINITY;
             if (a.num_splits > 1) {
                 const size_t prow = (size_t)bh * a.num_splits + split;  // Nq == 1
                 if (tid < d) a.O_partial[prow * d + tid] = o * inv;

@@ -573,7 +573,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     for (int nb = 0; nb < NB; ++nb) {
         const float l = xhalf_sum(l_run[nb]);
         const float inv = l > 0.0f ? (kDropout ? a.drop_rscale : 1.0f) / l : 0.0f;
-        const float lse = l > 0.0f ? (m_ref[nb] + fast_log2(l)) * kLn2 : -INFINITY;
+        const float lse = l > 0.0f ? __builtin_fmaf(m_ref[nb], kLn2, fast_log2(l) * kLn2) : -INFINITY;  // (one rounding at the size of m)
         const int i = row_i[nb];
         if (i >= Nq) continue;
         if (a.num_splits > 1) {

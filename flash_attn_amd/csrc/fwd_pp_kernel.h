@@ -509,7 +509,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     {
         const float l = xhalf_sum(l_run);
         const float inv = l > 0.0f ? (kDropout ? a.drop_rscale : 1.0f) / l : 0.0f;
-        const float lse = l > 0.0f ? (m_ref + fast_log2(l)) * kLn2 : -INFINITY;
+        const float lse = l > 0.0f ? __builtin_fmaf(m_ref, kLn2, fast_log2(l) * kLn2) : -INFINITY;
         if (a.num_splits > 1) {
             if (row_i < Nq) {
                 const size_t prow = ((size_t)bh * a.num_splits + split) * Nq + row_i;
