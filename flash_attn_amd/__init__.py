@@ -15,5 +15,10 @@ from .binding import (  # noqa: F401
     resolve_splits,
     workspace_bytes,
     library_path,
+    stage_stamp_names,
+    KERNEL_AUTO,
+    KERNEL_4WAVE,
+    KERNEL_8WAVE,
+    FLASH_STAMP_WORDS,
     lib,
 )

@@ -14,6 +14,8 @@ _LIB_PATH = os.path.join(_HERE, "lib", "libflash_attn_mi355.so")
 FLASH_OK = 0
 FLASH_MAX_HEAD_DIM = 128
 FLASH_MAX_SPLITS = 128
+FLASH_STAMP_WORDS = 8
+KERNEL_AUTO, KERNEL_4WAVE, KERNEL_8WAVE = 0, 1, 2
 
 
 class FlashError(RuntimeError):
@@ -39,6 +41,8 @@ class FlashParams(C.Structure):
         ("keep_mask_out", C.c_void_p),
         ("H_kv", C.c_int),
         ("scores_out", C.c_void_p),
+        ("kernel_hint", C.c_int),
+        ("stage_stamps_out", C.c_void_p),
     ]
 
 
@@ -73,6 +77,8 @@ def lib():
         L.flash_splitkv_workspace_bytes.argtypes = [pp, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
         L.flash_splitkv_resolve_splits.restype = C.c_int
         L.flash_splitkv_resolve_splits.argtypes = [pp]
+        L.flash_stage_stamps_bytes.restype = C.c_int
+        L.flash_stage_stamps_bytes.argtypes = [pp, C.c_int, C.POINTER(C.c_size_t)]
         L.flash_num_splits_heuristic.restype = C.c_int
         L.flash_num_splits_heuristic.argtypes = [C.c_int] * 5
         L.flash_dropout_keep_mask.restype = C.c_int
@@ -118,7 +124,7 @@ def _check_qkv(q, k, v):
 
 def make_params(q, k, v, o, lse, softmax_scale=None, causal=False, window=(-1, -1), alibi_slopes=None,
                 dropout_p=0.0, seed=0, offset=0, num_splits=1, o_partial=None, lse_partial=None, keep_mask_out=None,
-                scores_out=None):
+                scores_out=None, kernel_hint=KERNEL_AUTO):
     B, H, Nq, Nk, d = _check_qkv(q, k, v)
     p = FlashParams()
     p.Q, p.K, p.V, p.O, p.LSE = _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse)
@@ -134,15 +140,35 @@ def make_params(q, k, v, o, lse, softmax_scale=None, causal=False, window=(-1, -
     p.keep_mask_out = _ptr(keep_mask_out)
     p.H_kv = int(k.shape[1])
     p.scores_out = _ptr(scores_out)
+    p.kernel_hint = int(kernel_hint)
     return p
 
 
+def _attach_stamps(p, split, device):
+    """Allocates the stage-stamp buffer of the call described by p ([work-groups, FLASH_STAMP_WORDS] int64) and points
+    p at it; None when the call runs no tiled kernel."""
+    import torch
+
+    nb = C.c_size_t()
+    rc = lib().flash_stage_stamps_bytes(C.byref(p), int(split), C.byref(nb))
+    if rc != FLASH_OK:
+        raise FlashError(rc, "flash_stage_stamps_bytes")
+    if nb.value == 0:
+        return None
+    st = torch.zeros((nb.value // (8 * FLASH_STAMP_WORDS), FLASH_STAMP_WORDS), dtype=torch.int64, device=device)
+    p.stage_stamps_out = st.data_ptr()
+    return st
+
+
 def flash_forward(q, k, v, softmax_scale=None, causal=False, window=(-1, -1), alibi_slopes=None, dropout_p=0.0,
-                  seed=0, offset=0, return_keep_mask=False, stream=None, out=None, lse=None, scores_out=None):
+                  seed=0, offset=0, return_keep_mask=False, stream=None, out=None, lse=None, scores_out=None,
+                  kernel_hint=KERNEL_AUTO, return_stage_stamps=False):
     """O = softmax(mask(Q K^T * scale - slope * |i - j|)) V over the whole key range.
     q [B,H,Nq,d], k,v [B,H,Nk,d] fp16 on the GPU.  Returns (O fp16 [B,H,Nq,d], LSE fp32 [B,H,Nq]) and, when
     return_keep_mask, the uint8 keep decisions [B,H,Nq,Nk] the kernel applied.  scores_out: optional fp32
-    [B,H,Nq,Nk] tensor (pre-filled with -inf) that receives the visible scores (debug; slow kernel instance)."""
+    [B,H,Nq,Nk] tensor (pre-filled with -inf) that receives the visible scores (debug; slow kernel instance).
+    kernel_hint: KERNEL_AUTO / KERNEL_4WAVE / KERNEL_8WAVE.  return_stage_stamps: also return the per-work-group
+    time stamps [groups, 8] int64 of the instrumented kernel instance (debug), as the last element."""
     import torch
 
     B, H, Nq, Nk, d = _check_qkv(q, k, v)
@@ -150,41 +176,63 @@ def flash_forward(q, k, v, softmax_scale=None, causal=False, window=(-1, -1), al
     l = lse if lse is not None else torch.empty((B, H, Nq), dtype=torch.float32, device=q.device)
     km = torch.zeros((B, H, Nq, Nk), dtype=torch.uint8, device=q.device) if return_keep_mask else None
     p = make_params(q, k, v, o, l, softmax_scale, causal, window, alibi_slopes, dropout_p, seed, offset, 1,
-                    keep_mask_out=km, scores_out=scores_out)
+                    keep_mask_out=km, scores_out=scores_out, kernel_hint=kernel_hint)
+    stamps = _attach_stamps(p, 0, q.device) if return_stage_stamps else None
     rc = lib().flash_forward(C.byref(p), _stream_handle(stream))
     if rc != FLASH_OK:
         raise FlashError(rc, "flash_forward")
-    return (o, l, km) if return_keep_mask else (o, l)
+    res = (o, l, km) if return_keep_mask else (o, l)
+    return res + (stamps,) if return_stage_stamps else res
 
 
 def flash_forward_splitkv(q, k, v, num_splits=0, softmax_scale=None, causal=False, window=(-1, -1),
                           alibi_slopes=None, dropout_p=0.0, seed=0, offset=0, stream=None, workspace=None,
-                          return_partials=False, out=None, lse=None, scores_out=None):
-    """Split-KV forward + combine.  num_splits <= 0 asks the library's heuristic.  `workspace` may carry a
-    pre-allocated (O_partial, LSE_partial) pair; otherwise it is allocated here (the caller owns the workspace, as
-    in src/main.cu:160-162)."""
+                          return_partials=False, out=None, lse=None, scores_out=None, kernel_hint=KERNEL_AUTO,
+                          return_stage_stamps=False):
+    """Split-KV forward + combine.  num_splits <= 0 asks the library's heuristic; a larger request than there are
+    128-key blocks is clamped by the library (flash_splitkv_resolve_splits tells the count used).  `workspace` may
+    carry a pre-allocated (O_partial, LSE_partial) pair with at least the bytes flash_splitkv_workspace_bytes
+    reports; otherwise it is allocated here (the caller owns the workspace, as in src/main.cu:160-162).
+    return_partials hands back views of the workspace in the layout the library wrote, for the resolved split count
+    S: [B,H,S,Nq,d] / [B,H,S,Nq], or -- one query row with four or more query heads per K/V head, no ALiBi, left
+    window or dropout -- [B,H_kv,S,G,d] / [B,H_kv,S,G] with G = H / H_kv; (None, None) when S == 1."""
     import torch
 
     B, H, Nq, Nk, d = _check_qkv(q, k, v)
     o = out if out is not None else torch.empty((B, H, Nq, d), dtype=torch.float16, device=q.device)
     l = lse if lse is not None else torch.empty((B, H, Nq), dtype=torch.float32, device=q.device)
     p = make_params(q, k, v, o, l, softmax_scale, causal, window, alibi_slopes, dropout_p, seed, offset, num_splits,
-                    scores_out=scores_out)
-    if workspace is None:
-        ob, lb = C.c_size_t(), C.c_size_t()
-        rc = lib().flash_splitkv_workspace_bytes(C.byref(p), C.byref(ob), C.byref(lb))
-        if rc != FLASH_OK:
-            raise FlashError(rc, "flash_splitkv_workspace_bytes")
-        S = lib().flash_splitkv_resolve_splits(C.byref(p))
-        if ob.value:
-            workspace = (torch.empty((B, H, S, Nq, d), dtype=torch.float32, device=q.device),
-                         torch.empty((B, H, S, Nq), dtype=torch.float32, device=q.device))
+                    scores_out=scores_out, kernel_hint=kernel_hint)
+    S = lib().flash_splitkv_resolve_splits(C.byref(p))
+    if S < 0:
+        raise FlashError(S, "flash_splitkv_resolve_splits")
+    rows = B * H * S * Nq if S > 1 else 0
+    if workspace is None and rows:
+        workspace = (torch.empty(rows * d, dtype=torch.float32, device=q.device),
+                     torch.empty(rows, dtype=torch.float32, device=q.device))
     if workspace is not None:
+        if workspace[0].numel() < rows * d or workspace[1].numel() < rows:
+            raise ValueError(f"workspace too small for {S} splits: need {rows * d} and {rows} fp32 elements")
+        for t in workspace:
+            if t.dtype != torch.float32 or not t.is_cuda or not t.is_contiguous():
+                raise ValueError("workspace tensors must be contiguous fp32 device tensors")
         p.O_partial, p.LSE_partial = _ptr(workspace[0]), _ptr(workspace[1])
+    stamps = _attach_stamps(p, 1, q.device) if return_stage_stamps else None
     rc = lib().flash_forward_splitkv(C.byref(p), _stream_handle(stream))
     if rc != FLASH_OK:
         raise FlashError(rc, "flash_forward_splitkv")
-    return (o, l, workspace) if return_partials else (o, l)
+    res = (o, l)
+    if return_partials:
+        if rows:
+            Hk = k.shape[1]
+            G = H // Hk
+            grouped = (Nq == 1 and G >= 4 and alibi_slopes is None and not (0 <= window[0] < Nk) and dropout_p == 0.0
+                       and scores_out is None)
+            shp = (B, Hk, S, G) if grouped else (B, H, S, Nq)
+            res += ((workspace[0].reshape(-1)[:rows * d].view(*shp, d), workspace[1].reshape(-1)[:rows].view(*shp)),)
+        else:
+            res += ((None, None),)
+    return res + (stamps,) if return_stage_stamps else res
 
 
 def dropout_keep_mask(B, H, Nq, Nk, dropout_p, seed, offset=0, device="cuda", stream=None):
@@ -207,6 +255,12 @@ def dropout_threshold(p):
 
 def num_splits_heuristic(batch_nheads_mblocks, num_cus, num_n_blocks, max_splits, seq_len):
     return lib().flash_num_splits_heuristic(batch_nheads_mblocks, num_cus, num_n_blocks, max_splits, seq_len)
+
+
+def stage_stamp_names():
+    """Meaning of the eight words of a stage-stamp row (see stage_stamps_out in the header)."""
+    return ("entry", "requests_issued", "requests_landed", "first_barrier", "first_scores", "loop_done", "stored",
+            "tiles<<32|xcc<<16|hw_id")
 
 
 def _shape_params(B, H, Nq, Nk, d, num_splits):

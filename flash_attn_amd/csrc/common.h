@@ -35,6 +35,7 @@ struct FwdArgs {
     const float* alibi;  // [H] or nullptr
     uint8_t* keep_out;   // [B,H,Nq,Nk] or nullptr
     float* scores_out;   // [B,H,Nq,Nk] or nullptr (element-wise instance of the 4-wave kernel only)
+    uint64_t* stamps;    // [work-groups][kStampWords] or nullptr (instrumented instances only)
     int B, H, Nq, Nk, d;
     int Hk, kv_group;    // K/V heads and query heads per K/V head (H = Hk * kv_group)
     int causal, wl, wr;  // wl / wr < 0: unbounded
@@ -45,6 +46,7 @@ struct FwdArgs {
     int num_splits;      // 1: write O/LSE; > 1: write the partial workspace
     int keys_per_split;  // multiple of 128
     int Tr;              // number of query row blocks
+    int kernel_hint;     // 0: by shape, 1: 4-wave kernel, 2: 8-wave kernel where it can serve the call
 
     // index of the K/V slice [Nk,d] read by query slice bh = b * H + h
     __device__ __forceinline__ int kv_slice(int bh) const { return (bh / H) * Hk + (bh % H) / kv_group; }
@@ -64,6 +66,46 @@ __device__ __forceinline__ float xhalf_sum(float v)
     auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
+
+// Debug time stamps of the instrumented kernel instances: readings of the constant 100 MHz counter, taken by every wave
+// (they are scalar) and stored by the first lane of the work-group in the epilogue with an ordinary vector store.
+constexpr int kStampWords = 8;  // FLASH_STAMP_WORDS of the public header
+template <bool kOn>
+struct Stamps {
+    uint64_t t[kOn ? kStampWords - 1 : 1];
+    // stage 0 also presets the later stages: one that a work-group never reaches (no key tile) is stored as the time
+    // of the stage before it
+    __device__ __forceinline__ void take(int i)
+    {
+        if constexpr (kOn) {
+            const uint64_t now = __builtin_amdgcn_s_memrealtime();
+            if (i == 0) {
+#pragma unroll
+                for (int k = 0; k < kStampWords - 1; ++k) t[k] = now;
+            } else {
+                t[i] = now;
+            }
+        }
+    }
+    // word 7: tiles << 32 | XCC id << 16 | low half of HW_ID (wave, SIMD, pipe, CU, SH, SE)
+    __device__ __forceinline__ void store(uint64_t* out, int ntiles) const
+    {
+        if constexpr (kOn) {
+            if (out != nullptr && threadIdx.x == 0) {
+                const uint32_t hw = __builtin_amdgcn_s_getreg((31 << 11) | 4);    // HW_REG_HW_ID
+                const uint32_t xcc = __builtin_amdgcn_s_getreg((31 << 11) | 20);  // HW_REG_XCC_ID
+                uint64_t* o = out + (size_t)blockIdx.x * kStampWords;
+                uint64_t last = t[0];
+#pragma unroll
+                for (int i = 0; i < kStampWords - 1; ++i) {
+                    last = t[i] > last ? t[i] : last;
+                    o[i] = last;
+                }
+                o[kStampWords - 1] = ((uint64_t)(uint32_t)ntiles << 32) | ((uint64_t)(xcc & 0xfu) << 16) | (hw & 0xffffu);
+            }
+        }
+    }
+};
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
@@ -118,6 +160,18 @@ __device__ __forceinline__ void dma_kib(const char* base, uint32_t off, FA_LDS c
                  :
                  : "s"(m0v), "v"(off), "s"(base)
                  : "memory", "m0");
+}
+
+// Launch with the error of THIS launch as the return value (hipGetLastError would also hand back whatever an
+// unrelated earlier call of the process left behind).
+template <typename T>
+struct same_type { typedef T type; };
+template <typename... P>
+inline hipError_t launch_kernel(void (*kern)(P...), dim3 grid, dim3 block, size_t smem, hipStream_t st,
+                                typename same_type<P>::type... args)
+{
+    void* argv[] = {static_cast<void*>(&args)...};
+    return hipLaunchKernel(reinterpret_cast<const void*>(kern), grid, block, argv, smem, st);
 }
 
 // Raises the dynamic-LDS limit of a kernel once per device (the attribute belongs to the device's copy of the kernel).

@@ -244,38 +244,36 @@ __global__ void __launch_bounds__(256) keep_mask_kernel(uint8_t* __restrict__ ma
 }
 
 template <int LPK, int G>
-static void launch_decode_instance(const FwdArgs& a, hipStream_t st)
+static hipError_t launch_decode_instance(const FwdArgs& a, hipStream_t st)
 {
     const unsigned groups = (unsigned)((long long)a.B * a.H / G * a.num_splits);
-    if (a.alibi != nullptr) hipLaunchKernelGGL((decode_split_kernel<LPK, true, G>), dim3(groups), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((decode_split_kernel<LPK, false, G>), dim3(groups), dim3(256), 0, st, a);
+    if (a.alibi != nullptr) return launch_kernel(decode_split_kernel<LPK, true, G>, dim3(groups), dim3(256), 0, st, a);
+    return launch_kernel(decode_split_kernel<LPK, false, G>, dim3(groups), dim3(256), 0, st, a);
 }
 
 template <int LPK>
-static void launch_decode_bucket(const FwdArgs& a, hipStream_t st)
+static hipError_t launch_decode_bucket(const FwdArgs& a, hipStream_t st)
 {
     // as many of the query heads of a K/V head per work-group as divide the group (up to 8)
-    if (a.kv_group % 8 == 0) launch_decode_instance<LPK, 8>(a, st);
-    else if (a.kv_group % 4 == 0) launch_decode_instance<LPK, 4>(a, st);
-    else if (a.kv_group % 2 == 0) launch_decode_instance<LPK, 2>(a, st);
-    else launch_decode_instance<LPK, 1>(a, st);
+    if (a.kv_group % 8 == 0) return launch_decode_instance<LPK, 8>(a, st);
+    if (a.kv_group % 4 == 0) return launch_decode_instance<LPK, 4>(a, st);
+    if (a.kv_group % 2 == 0) return launch_decode_instance<LPK, 2>(a, st);
+    return launch_decode_instance<LPK, 1>(a, st);
 }
 
 int launch_decode_split(const FwdArgs& a, hipStream_t st)
 {
-    if (a.d > 64) launch_decode_bucket<16>(a, st);
-    else if (a.d > 32) launch_decode_bucket<8>(a, st);
-    else launch_decode_bucket<4>(a, st);
-    return (int)hipGetLastError();
+    if (a.d > 64) return (int)launch_decode_bucket<16>(a, st);
+    if (a.d > 32) return (int)launch_decode_bucket<8>(a, st);
+    return (int)launch_decode_bucket<4>(a, st);
 }
 
 int launch_combine(const FwdArgs& a, hipStream_t st)
 {
     const long long rows = (long long)a.B * a.H * a.Nq;
     const unsigned groups = (unsigned)((rows + 3) / 4);
-    hipLaunchKernelGGL(combine_kernel, dim3(groups), dim3(256), 0, st, a.O_partial, a.LSE_partial, a.O, a.LSE,
-                       a.B * a.H, a.Nq, a.d, a.num_splits);
-    return (int)hipGetLastError();
+    return (int)launch_kernel(combine_kernel, dim3(groups), dim3(256), 0, st, a.O_partial, a.LSE_partial, a.O, a.LSE,
+                              a.B * a.H, a.Nq, a.d, a.num_splits);
 }
 
 int launch_keep_mask(uint8_t* mask, int B, int H, int Nq, int Nk, uint32_t thr, uint64_t seed, uint64_t offset,
@@ -286,9 +284,8 @@ int launch_keep_mask(uint8_t* mask, int B, int H, int Nq, int Nk, uint32_t thr, 
     long long groups = (total + 255) / 256;
     if (groups > 65536) groups = 65536;
     if (groups < 1) groups = 1;
-    hipLaunchKernelGGL(keep_mask_kernel, dim3((unsigned)groups), dim3(256), 0, st, mask, rows, Nq, Nk, thr,
-                       (uint32_t)seed, (uint32_t)(seed >> 32), (uint32_t)offset);
-    return (int)hipGetLastError();
+    return (int)launch_kernel(keep_mask_kernel, dim3((unsigned)groups), dim3(256), 0, st, mask, rows, Nq, Nk, thr,
+                              (uint32_t)seed, (uint32_t)(seed >> 32), (uint32_t)offset);
 }
 
 }  // namespace fa

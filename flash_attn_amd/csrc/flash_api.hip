@@ -3,6 +3,7 @@
 // arguments, pick the kernel, size the grid, enqueue (+ combine when the key range is split).
 #include "flash_attn_mi355.h"
 
+#include <atomic>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -26,6 +27,24 @@ int record_hip(int e)
 
 constexpr int kNumCU = 256;  // MI355X
 
+// The library carries gfx950 code only: on any other device the first launch would fail with a HIP error that says
+// little.  Checked once per device (0 = not yet, 1 = gfx950, 2 = something else).
+int device_usable()
+{
+    static std::atomic<int> state[fa::kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return FLASH_ENODEVICE;
+    const bool cached = dev >= 0 && dev < fa::kMaxDevices;
+    int st = cached ? state[dev].load(std::memory_order_relaxed) : 0;
+    if (st == 0) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return FLASH_ENODEVICE;
+        st = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 2;
+        if (cached) state[dev].store(st, std::memory_order_relaxed);
+    }
+    return st == 1 ? FLASH_OK : FLASH_ENODEVICE;
+}
+
 inline bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
 
 // shape / scalar checks shared by every entry point; *empty is set when there is nothing to compute
@@ -40,10 +59,12 @@ int validate_shape(const flash_params* p, bool* empty)
     if (p->num_splits > FLASH_MAX_SPLITS) return FLASH_ESPLITS;
     if ((long long)p->B * p->H > 0x7fffffffLL / 2) return FLASH_EINVAL;
     // one-dimensional grids: slices x row blocks x splits must fit the 2^31 - 1 work-groups of a launch
-    if ((long long)p->B * p->H * ((p->Nq + 127) / 128) > 0x7fffffffLL / FLASH_MAX_SPLITS) return FLASH_EINVAL;
+    if ((long long)p->B * p->H * (((long long)p->Nq + 127) / 128) > 0x7fffffffLL / FLASH_MAX_SPLITS) return FLASH_EINVAL;
+    if ((long long)p->Nq + p->Nk > 0x7fffffffLL) return FLASH_EINVAL;  // row + window arithmetic stays in int
     // the tile requests address a [N,d] slice with 32-bit byte offsets
     if (2LL * p->Nq * p->d >= (1LL << 32) || 2LL * p->Nk * p->d >= (1LL << 32)) return FLASH_EINVAL;
     if (p->H_kv < 0 || (p->H_kv > 0 && (p->H_kv > p->H || p->H % p->H_kv != 0))) return FLASH_EINVAL;
+    if (p->kernel_hint < 0 || p->kernel_hint > 2) return FLASH_EINVAL;
     if (p->B == 0 || p->H == 0 || p->Nq == 0) *empty = true;
     return FLASH_OK;
 }
@@ -61,6 +82,7 @@ int validate(const flash_params* p, bool* empty)
     if (p->Nk > 0 && (misaligned(p->K, need) || misaligned(p->V, need))) return FLASH_EALIGN;
     if (p->alibi_slopes && misaligned(p->alibi_slopes, 4)) return FLASH_EALIGN;
     if (p->scores_out && misaligned(p->scores_out, 4)) return FLASH_EALIGN;
+    if (p->stage_stamps_out && misaligned(p->stage_stamps_out, 8)) return FLASH_EALIGN;
     return FLASH_OK;
 }
 
@@ -79,6 +101,8 @@ void fill_args(const flash_params* p, int splits, fa::FwdArgs* a)
     a->alibi = p->alibi_slopes;
     a->keep_out = p->dropout_p > 0.0f ? p->keep_mask_out : nullptr;
     a->scores_out = p->scores_out;
+    a->stamps = p->stage_stamps_out;
+    a->kernel_hint = p->kernel_hint;
     a->B = p->B;
     a->H = p->H;
     a->Nq = p->Nq;
@@ -87,8 +111,10 @@ void fill_args(const flash_params* p, int splits, fa::FwdArgs* a)
     a->Hk = p->H_kv > 0 ? p->H_kv : (p->H > 0 ? p->H : 1);
     a->kv_group = p->H > 0 ? p->H / a->Hk : 1;
     a->causal = p->is_causal ? 1 : 0;
-    a->wl = p->window_left;
-    a->wr = p->window_right;
+    // A bound that can never cut (i' - j <= Nk - 1, j - i' <= Nq - 1 for the row index i' = i + Nk - Nq) is the same
+    // as no bound; callers write "unbounded" as INT_MAX too, which the kernels' i' + right would overflow.
+    a->wl = p->window_left >= p->Nk ? -1 : p->window_left;
+    a->wr = p->window_right >= p->Nq ? -1 : p->window_right;
     a->scale_log2 = p->softmax_scale * fa::kLog2e;
     a->drop_thr = flash_dropout_threshold(p->dropout_p);
     a->drop_rscale = 1.0f / (1.0f - p->dropout_p);
@@ -101,18 +127,34 @@ void fill_args(const flash_params* p, int splits, fa::FwdArgs* a)
     a->Tr = (p->Nq + kRowsPerGroup - 1) / kRowsPerGroup;
 }
 
-int launch_tiled(const flash_params* p, const fa::FwdArgs& a, hipStream_t st)
+// variant bits of the tiled kernel for p (kVarVec | kVarAlibi | kVarDropout of fwd_kernel.h)
+int tiled_variant(const flash_params* p)
 {
     // A non-positive scale does not commute with the row maximum: only the element-wise instance scales first.
     int variant = (p->d % 8 == 0 && p->softmax_scale > 0.0f && !p->scores_out) ? 1 : 0;  // (the score dump lives there too)
     if (p->alibi_slopes) variant |= 2;
     if (p->dropout_p > 0.0f) variant |= 4;
+    return variant;
+}
+
+int launch_tiled(const flash_params* p, const fa::FwdArgs& a, hipStream_t st)
+{
+    const int variant = tiled_variant(p);
     int e;
     if (p->d <= 32) e = fa::launch_fwd_d32(a, variant, 1, st);
     else if (p->d <= 64) e = fa::launch_fwd_d64(a, variant, 1, st);
     else if (p->d <= 96) e = fa::launch_fwd_d96(a, variant, 1, st);
     else e = fa::launch_fwd_d128(a, variant, 1, st);
     return record_hip(e);
+}
+
+// work-groups of the tiled launch for the (final) arguments a
+long long tiled_groups(const flash_params* p, const fa::FwdArgs& a)
+{
+    const bool pp = a.d > 96 && fa::fwd_uses_pingpong(a.d, (tiled_variant(p) & 1) != 0, a.Nq, a.causal, a.wl, a.wr,
+                                                      (long long)a.B * a.H * a.num_splits, a.kernel_hint);
+    const int rows = pp ? 256 : kRowsPerGroup;
+    return (long long)((a.Nq + rows - 1) / rows) * a.B * a.H * a.num_splits;
 }
 
 int resolve_splits(const flash_params* p)
@@ -135,7 +177,8 @@ int resolve_splits(const flash_params* p)
         s = (int)(want < by_keys ? want : by_keys);
     } else if (s <= 0) {
         const bool vec = p->d % 8 == 0 && p->softmax_scale > 0.0f;
-        const int rows = fa::fwd_uses_pingpong(p->d, vec, p->Nq, p->is_causal, p->window_left, p->window_right, (long long)p->B * p->H) ? 256 : kRowsPerGroup;
+        const int rows = fa::fwd_uses_pingpong(p->d, vec, p->Nq, p->is_causal, p->window_left, p->window_right,
+                                               (long long)p->B * p->H, p->kernel_hint) ? 256 : kRowsPerGroup;
         const int Tr = (p->Nq + rows - 1) / rows;
         // argument roles as in the reference's call (src/main.cu:125), with the CU count of the MI355X and the row
         // blocks of the kernel that will run
@@ -147,6 +190,31 @@ int resolve_splits(const flash_params* p)
     return s;
 }
 
+// Which kernel serves a split-KV call; may reshape the arguments (grouped decode).
+constexpr int kRouteTiled = 0, kRouteStream = 1;
+int splitkv_route(const flash_params* p, fa::FwdArgs* a)
+{
+    if (p->scores_out) return kRouteTiled;  // debug dump: element-wise instance of the tiled kernel
+    if (p->Nq == 1 && a->kv_group >= 4 && !p->alibi_slopes && a->wl < 0 && p->dropout_p == 0.0f) {
+        // Decode with grouped K/V heads: the G query heads of one K/V head, one row each, are the G rows of one
+        // attention problem over that K/V head -- Q [B,H,1,d] is [B,H_kv,G,d] in memory, and so are O, LSE and the
+        // split workspace.  The tiled kernel then streams K/V once per K/V head and does the arithmetic on the MFMA
+        // units (measured 1.4x - 4x faster than G dot products per key on the VALU for G = 8 ... 32, equal at G = 4).
+        // The single query row sits at position Nk - 1 and sees every key whatever the causal flag or the right
+        // window say; as rows of a G-row problem the heads must not get a mask that depends on the row.
+        a->H = a->Hk;
+        a->Nq = a->kv_group;
+        a->kv_group = 1;
+        a->causal = 0;
+        a->wr = -1;
+        a->Tr = (a->Nq + kRowsPerGroup - 1) / kRowsPerGroup;
+        return kRouteTiled;
+    }
+    // one query row per head, 16-byte rows, no dropout: bandwidth-bound streaming kernel
+    if (p->Nq == 1 && p->d % 8 == 0 && p->dropout_p == 0.0f && p->softmax_scale > 0.0f) return kRouteStream;
+    return kRouteTiled;
+}
+
 }  // namespace
 
 #define FLASH_EXPORT __attribute__((visibility("default")))
@@ -156,8 +224,9 @@ extern "C" {
 FLASH_EXPORT int flash_forward(const flash_params* p, void* stream)
 {
     bool empty;
-    const int rc = validate(p, &empty);
+    int rc = validate(p, &empty);
     if (rc != FLASH_OK || empty) return rc;
+    if ((rc = device_usable()) != FLASH_OK) return rc;
     fa::FwdArgs a;
     fill_args(p, 1, &a);
     return launch_tiled(p, a, static_cast<hipStream_t>(stream));
@@ -166,37 +235,33 @@ FLASH_EXPORT int flash_forward(const flash_params* p, void* stream)
 FLASH_EXPORT int flash_forward_splitkv(const flash_params* p, void* stream)
 {
     bool empty;
-    const int rc = validate(p, &empty);
+    int rc = validate(p, &empty);
     if (rc != FLASH_OK || empty) return rc;
     const int splits = resolve_splits(p);
     if (splits > 1 && (!p->O_partial || !p->LSE_partial)) return FLASH_EWORKSPACE;
     if (splits > 1 && (misaligned(p->O_partial, 16) || misaligned(p->LSE_partial, 4))) return FLASH_EALIGN;
+    if ((rc = device_usable()) != FLASH_OK) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
     fa::FwdArgs a;
     fill_args(p, splits, &a);
-    int e;
-    if (p->scores_out) {
-        e = launch_tiled(p, a, st);  // debug dump: element-wise instance of the tiled kernel
-    } else if (p->Nq == 1 && a.kv_group >= 4 && !p->alibi_slopes && p->window_left < 0 && p->dropout_p == 0.0f) {
-        // Decode with grouped K/V heads: the G query heads of one K/V head, one row each, are the G rows of one
-        // attention problem over that K/V head -- Q [B,H,1,d] is [B,H_kv,G,d] in memory, and so are O, LSE and the
-        // split workspace, and no mask depends on the row.  The tiled kernel then streams K/V once per K/V head and
-        // does the arithmetic on the MFMA units (measured 1.4x - 4x faster than G dot products per key on the VALU
-        // for G = 8 ... 32, equal at G = 4).
-        a.H = a.Hk;
-        a.Nq = a.kv_group;
-        a.kv_group = 1;
-        a.causal = 0;
-        a.Tr = (a.Nq + kRowsPerGroup - 1) / kRowsPerGroup;
-        e = launch_tiled(p, a, st);
-    } else if (p->Nq == 1 && p->d % 8 == 0 && p->dropout_p == 0.0f && p->softmax_scale > 0.0f) {
-        // one query row per head, 16-byte rows, no dropout: bandwidth-bound streaming kernel
-        e = record_hip(fa::launch_decode_split(a, st));
-    } else {
-        e = launch_tiled(p, a, st);
-    }
+    const int route = splitkv_route(p, &a);
+    const int e = route == kRouteStream ? record_hip(fa::launch_decode_split(a, st)) : launch_tiled(p, a, st);
     if (e != FLASH_OK || splits == 1) return e;
     return record_hip(fa::launch_combine(a, st));
+}
+
+FLASH_EXPORT int flash_stage_stamps_bytes(const flash_params* p, int split, size_t* bytes)
+{
+    if (!bytes) return FLASH_EINVAL;
+    *bytes = 0;
+    bool empty;
+    const int rc = validate_shape(p, &empty);
+    if (rc != FLASH_OK || empty) return rc;
+    fa::FwdArgs a;
+    fill_args(p, split ? resolve_splits(p) : 1, &a);
+    if (split && splitkv_route(p, &a) == kRouteStream) return FLASH_OK;
+    *bytes = (size_t)tiled_groups(p, a) * FLASH_STAMP_WORDS * sizeof(uint64_t);
+    return FLASH_OK;
 }
 
 FLASH_EXPORT int flash_splitkv_resolve_splits(const flash_params* p)
@@ -276,7 +341,7 @@ FLASH_EXPORT const char* flash_strerror(int code)
         case FLASH_EWORKSPACE: return "split workspace missing";
         case FLASH_ESPLITS: return "too many splits";
         case FLASH_ELAUNCH: return "HIP launch failed";
-        case FLASH_ENODEVICE: return "no usable gfx950 device";
+        case FLASH_ENODEVICE: return "the current device is not a gfx950";
         default: return "unknown error";
     }
 }

@@ -1,9 +1,7 @@
 // Instances of the tiled forward kernels for the head-dim bucket d <= 128.
-#include <cstdlib>
-
 #include "fwd_pp_kernel.h"
 namespace fa {
-bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr, long long slices)
+bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr, long long slices, int hint)
 {
     // d == 128, more than one 128-row block of queries and no narrow window: the 8-wave ping-pong kernel (measured
     // 3-18 % faster than the 4-wave kernel there; slower for d = 64 and for windows much smaller than its 256-row
@@ -12,13 +10,11 @@ bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr, long
     // share of the work (measured 4-9 % slower over B*H = 8 ... 1024 at N = 512 and 1024).  And with one 8-wave
     // work-group per CU its grid should make at least two full rounds of the 256 CUs: below that the 4-wave kernel
     // (two work-groups of half the rows per CU) fills the chip better (measured +4 ... +13 %, one shape -8 %).
-    // FLASH_ATTN_KERNEL=4wave / =8wave (read at every call) overrides these preferences for A/B runs and tests; the
-    // 8-wave kernel still needs d == 128 in whole 16-byte rows and more than 128 query rows.
+    // The caller's hint (flash_params::kernel_hint: 1 = 4-wave, 2 = 8-wave) overrides these preferences for A/B runs
+    // and tests; the 8-wave kernel still needs d == 128 in whole 16-byte rows and more than 128 query rows.
     const bool able = vec && d == 128 && Nq > 128;
-    if (const char* force = std::getenv("FLASH_ATTN_KERNEL")) {
-        if (force[0] == '4') return false;
-        if (force[0] == '8') return able;
-    }
+    if (hint == 1) return false;
+    if (hint == 2) return able;
     const bool narrow_window = (wl >= 0 && wl < 512) || (wr >= 0 && wr < 512 && !causal);
     const bool short_causal = causal && Nq <= 1024;
     const long long groups = slices * ((Nq + 255) / 256);
@@ -28,7 +24,8 @@ bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr, long
 int launch_fwd_d128(const FwdArgs& a, int variant, int nb, hipStream_t st)
 {
     (void)nb;
-    if (fwd_uses_pingpong(a.d, (variant & kVarVec) != 0, a.Nq, a.causal, a.wl, a.wr, (long long)a.B * a.H * a.num_splits))
+    if (fwd_uses_pingpong(a.d, (variant & kVarVec) != 0, a.Nq, a.causal, a.wl, a.wr, (long long)a.B * a.H * a.num_splits,
+                          a.kernel_hint))
         return launch_fwd_pp_bucket<128>(a, variant, st);
     return launch_fwd_bucket<128, 1>(a, variant, st);
 }

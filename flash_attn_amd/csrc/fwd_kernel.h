@@ -91,14 +91,16 @@ __device__ __forceinline__ v4u load_chunk(const half_t* __restrict__ rowp, int c
 constexpr float kLazyTau = 8.0f;
 
 // variant bits of the kernel template
-constexpr int kVarVec = 1, kVarAlibi = 2, kVarDropout = 4, kVarFullD = 8;
+constexpr int kVarVec = 1, kVarAlibi = 2, kVarDropout = 4, kVarFullD = 8, kVarStamp = 16;  // kVarStamp: debug time stamps
 
 template <int D, int NB, int VAR>
 __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 0 ? 3 : 2) : 1) fwd_kernel(const FwdArgs a)
 {
     constexpr bool kVec = (VAR & kVarVec) != 0, kAlibi = (VAR & kVarAlibi) != 0, kDropout = (VAR & kVarDropout) != 0,
-                   kFullD = (VAR & kVarFullD) != 0;
+                   kFullD = (VAR & kVarFullD) != 0, kStamp = (VAR & kVarStamp) != 0;
     using C = FwdCfg<D, NB>;
+    Stamps<kStamp> stamps;
+    stamps.take(0);
     constexpr int BC = C::BC, KS = C::KS, MB = C::MB, CH = C::CH, SK = C::SK, SV = C::SV, NLD = C::NLD;
     constexpr bool kDma = C::DMA && kVec && kFullD && (D >= 128 || !kDropout);
     constexpr int NSTG = kDma ? C::NSTG : 2;
@@ -529,14 +531,18 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
 #pragma unroll
         for (int u = 0; u < PF; ++u)
             if (u < ntiles) dma_tile(tile_begin + u, u);
+        stamps.take(1);
         dma_wait(PF == 2 && ntiles > 1);
         pin_q();
+        stamps.take(2);
         __syncthreads();
+        stamps.take(3);
         int buf = 0, nbuf = PF % NSTG;  // stages of tile t and of tile t + PF
         for (int t = 0; t < ntiles; ++t) {
             const bool more = t + PF < ntiles;
             if (more) dma_tile(tile_begin + t + PF, nbuf);
             tile_math(t, buf);
+            if (kStamp && t == 0) stamps.take(4);
             dma_wait(PF == 2 && more);
             __syncthreads();
             buf = buf + 1 == NSTG ? 0 : buf + 1;
@@ -547,11 +553,14 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
         if (ntiles > 0) {
             gload(Kbh, tile_begin, kreg);
             gload(Vbh, tile_begin, vreg);
+            stamps.take(1);
             put_k(0);
             put_v(0);
         }
         pin_q();
+        stamps.take(2);
         __syncthreads();
+        stamps.take(3);
         for (int t = 0; t < ntiles; ++t) {
             const int cur = t & 1;
             const bool has1 = t + 1 < ntiles;
@@ -560,6 +569,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                 gload(Vbh, tile_begin + t + 1, vreg);
             }
             tile_math(t, cur);
+            if (kStamp && t == 0) stamps.take(4);
             if (has1) {
                 put_k(cur ^ 1);
                 put_v(cur ^ 1);
@@ -569,6 +579,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     }
 
     // ---------------- epilogue: normalise once, store O (fp16) + LSE, or the fp32 split partials
+    stamps.take(5);
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         const float l = xhalf_sum(l_run[nb]);
@@ -649,6 +660,11 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
             }
         }
     }
+    if constexpr (kStamp) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the result stores of this wave have left
+        stamps.take(6);
+        stamps.store(a.stamps, ntiles);
+    }
 }
 
 // Launcher of one head-dim bucket, defined in fwd_d{32,64,96,128}.hip.
@@ -658,8 +674,8 @@ int launch_fwd_d64(const FwdArgs& a, int variant, int nb, hipStream_t st);
 int launch_fwd_d96(const FwdArgs& a, int variant, int nb, hipStream_t st);
 int launch_fwd_d128(const FwdArgs& a, int variant, int nb, hipStream_t st);
 // whether launch_fwd_d128 takes the 8-wave kernel (256 query rows per work-group instead of 128)
-// (slices = B * H * num_splits)
-bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr, long long slices);
+// (slices = B * H * num_splits; hint = flash_params::kernel_hint)
+bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr, long long slices, int hint);
 
 template <int D, int NB, int VAR>
 inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
@@ -670,32 +686,37 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
     constexpr int smem = C::SMEM_DMA > C::SMEM ? C::SMEM_DMA : C::SMEM;  // (equal: both paths use two stages)
     if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, attr_done); e != hipSuccess) return e;
     const long long groups = (long long)a.Tr * a.B * a.H * a.num_splits;
-    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(256), smem, st, a);
-    return hipGetLastError();
+    return launch_kernel(kern, dim3((unsigned)groups), dim3(256), smem, st, a);
 }
 
 // The nine instances of a bucket: {d == bucket, d % 8 == 0} x {plain, ALiBi, dropout, both}, and the element-wise
 // path with both features compiled in (slope 0 / threshold 0 make them identities, so it serves every request
-// with d % 8 != 0).
-template <int D, int NB>
-inline int launch_fwd_bucket(const FwdArgs& a, int variant, hipStream_t st)
+// with d % 8 != 0).  ST = kVarStamp selects their instrumented twins (debug time stamps).
+template <int D, int NB, int ST>
+inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
 {
     hipError_t e;
     const int feat = variant & (kVarAlibi | kVarDropout);
     if (!(variant & kVarVec)) {
-        e = launch_fwd_instance<D, NB, kVarAlibi | kVarDropout>(a, st);
+        e = launch_fwd_instance<D, NB, ST | kVarAlibi | kVarDropout>(a, st);
     } else if (a.d == D) {
-        if (feat == 0) e = launch_fwd_instance<D, NB, kVarVec | kVarFullD>(a, st);
-        else if (feat == kVarAlibi) e = launch_fwd_instance<D, NB, kVarVec | kVarFullD | kVarAlibi>(a, st);
-        else if (feat == kVarDropout) e = launch_fwd_instance<D, NB, kVarVec | kVarFullD | kVarDropout>(a, st);
-        else e = launch_fwd_instance<D, NB, kVarVec | kVarFullD | kVarAlibi | kVarDropout>(a, st);
+        if (feat == 0) e = launch_fwd_instance<D, NB, ST | kVarVec | kVarFullD>(a, st);
+        else if (feat == kVarAlibi) e = launch_fwd_instance<D, NB, ST | kVarVec | kVarFullD | kVarAlibi>(a, st);
+        else if (feat == kVarDropout) e = launch_fwd_instance<D, NB, ST | kVarVec | kVarFullD | kVarDropout>(a, st);
+        else e = launch_fwd_instance<D, NB, ST | kVarVec | kVarFullD | kVarAlibi | kVarDropout>(a, st);
     } else {
-        if (feat == 0) e = launch_fwd_instance<D, NB, kVarVec>(a, st);
-        else if (feat == kVarAlibi) e = launch_fwd_instance<D, NB, kVarVec | kVarAlibi>(a, st);
-        else if (feat == kVarDropout) e = launch_fwd_instance<D, NB, kVarVec | kVarDropout>(a, st);
-        else e = launch_fwd_instance<D, NB, kVarVec | kVarAlibi | kVarDropout>(a, st);
+        if (feat == 0) e = launch_fwd_instance<D, NB, ST | kVarVec>(a, st);
+        else if (feat == kVarAlibi) e = launch_fwd_instance<D, NB, ST | kVarVec | kVarAlibi>(a, st);
+        else if (feat == kVarDropout) e = launch_fwd_instance<D, NB, ST | kVarVec | kVarDropout>(a, st);
+        else e = launch_fwd_instance<D, NB, ST | kVarVec | kVarAlibi | kVarDropout>(a, st);
     }
     return (int)e;
+}
+
+template <int D, int NB>
+inline int launch_fwd_bucket(const FwdArgs& a, int variant, hipStream_t st)
+{
+    return a.stamps ? launch_fwd_bucket_st<D, NB, kVarStamp>(a, variant, st) : launch_fwd_bucket_st<D, NB, 0>(a, variant, st);
 }
 
 }  // namespace fa

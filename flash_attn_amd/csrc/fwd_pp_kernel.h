@@ -68,8 +68,10 @@ __device__ __forceinline__ void lds_barrier_keep(void)
 template <int D, int VAR>
 __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
 {
-    constexpr bool kAlibi = (VAR & kVarAlibi) != 0, kDropout = (VAR & kVarDropout) != 0;
+    constexpr bool kAlibi = (VAR & kVarAlibi) != 0, kDropout = (VAR & kVarDropout) != 0, kStamp = (VAR & kVarStamp) != 0;
     using C = PPCfg<D>;
+    Stamps<kStamp> stamps;
+    stamps.take(0);
     constexpr int BC = C::BC, KS = C::KS, MB = C::MB, NKL = C::NKL, NVL = C::NVL, NST = C::NST;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     FA_LDS char* const Ks = (FA_LDS char*)smem;
@@ -468,7 +470,9 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
             }
             if (ntiles > 2) load_k(2, Ks + 2 * C::KBUF);
         }
+        stamps.take(1);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (a memory clobber: the reads below stay below)
+        stamps.take(2);
         const uint32_t qbase = (uint32_t)(uintptr_t)qst + (uint32_t)k_rd;  // same lane part as a K fragment
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
@@ -478,7 +482,16 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));  // Q is in registers before the loop
     lds_barrier();  // tiles visible to all waves; every wave has read its Q rows (their LDS is reused by the loop)
-    if (ntiles > 0) qk(Ks);
+    stamps.take(3);
+    if (ntiles > 0) {
+        qk(Ks);
+        if constexpr (kStamp) {
+            // reading a score back makes the wave wait for the last MFMA before the stamp is taken
+            const int done = __builtin_amdgcn_readfirstlane(__float_as_int(s[1][15]));
+            asm volatile("; first scores are there" ::"s"(done));
+            stamps.take(4);
+        }
+    }
     if (grp == 1) lds_barrier();  // second wave group runs half an iteration behind
 
     // Tiles whose keys (and whose successor's keys) are all invisible to this wave contribute nothing: there the wave
@@ -504,6 +517,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
                   Vs + ((t + 2) % NST) * C::VBUF, t);
     for (; t < ntiles; ++t) idle_iteration(t);
     if (grp == 0) lds_barrier();  // both groups pass the same number of barriers
+    stamps.take(5);
 
     // ---------------- epilogue
     {
@@ -553,6 +567,11 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
             }
         }
     }
+    if constexpr (kStamp) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the result stores of this wave have left
+        stamps.take(6);
+        stamps.store(a.stamps, ntiles);
+    }
 }
 
 template <int D, int VAR>
@@ -565,21 +584,26 @@ inline hipError_t launch_fwd_pp_instance(const FwdArgs& a, hipStream_t st)
     FwdArgs b = a;
     b.Tr = (a.Nq + C::BR - 1) / C::BR;
     const long long groups = (long long)b.Tr * a.B * a.H * a.num_splits;
-    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(512), C::SMEM, st, b);
-    return hipGetLastError();
+    return launch_kernel(kern, dim3((unsigned)groups), dim3(512), C::SMEM, st, b);
 }
 
-// d == D, 16-byte rows: {plain, ALiBi, dropout, both}
-template <int D>
-inline int launch_fwd_pp_bucket(const FwdArgs& a, int variant, hipStream_t st)
+// d == D, 16-byte rows: {plain, ALiBi, dropout, both}; ST = kVarStamp: their instrumented twins
+template <int D, int ST>
+inline int launch_fwd_pp_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
 {
     const int feat = variant & (kVarAlibi | kVarDropout);
     hipError_t e;
-    if (feat == 0) e = launch_fwd_pp_instance<D, 0>(a, st);
-    else if (feat == kVarAlibi) e = launch_fwd_pp_instance<D, kVarAlibi>(a, st);
-    else if (feat == kVarDropout) e = launch_fwd_pp_instance<D, kVarDropout>(a, st);
-    else e = launch_fwd_pp_instance<D, kVarAlibi | kVarDropout>(a, st);
+    if (feat == 0) e = launch_fwd_pp_instance<D, ST>(a, st);
+    else if (feat == kVarAlibi) e = launch_fwd_pp_instance<D, ST | kVarAlibi>(a, st);
+    else if (feat == kVarDropout) e = launch_fwd_pp_instance<D, ST | kVarDropout>(a, st);
+    else e = launch_fwd_pp_instance<D, ST | kVarAlibi | kVarDropout>(a, st);
     return (int)e;
+}
+
+template <int D>
+inline int launch_fwd_pp_bucket(const FwdArgs& a, int variant, hipStream_t st)
+{
+    return a.stamps ? launch_fwd_pp_bucket_st<D, kVarStamp>(a, variant, st) : launch_fwd_pp_bucket_st<D, 0>(a, variant, st);
 }
 
 }  // namespace fa

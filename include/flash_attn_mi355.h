@@ -28,7 +28,7 @@ enum {
     FLASH_EWORKSPACE = -4,   /* num_splits > 1 but O_partial / LSE_partial missing                           */
     FLASH_ESPLITS = -5,      /* num_splits larger than FLASH_MAX_SPLITS                                      */
     FLASH_ELAUNCH = -6,      /* the HIP runtime rejected a launch; see flash_last_hip_error()                */
-    FLASH_ENODEVICE = -7     /* no gfx950 device / code object not loadable on the current device           */
+    FLASH_ENODEVICE = -7     /* the current device is not a gfx950 (the library carries code for nothing else) */
 };
 
 #define FLASH_MAX_HEAD_DIM 128
@@ -86,7 +86,23 @@ typedef struct flash_params {
      * as the masked score matrix).  The call then takes the element-wise kernel instance, which serves every
      * feature but is several times slower.  No counterpart in the reference. */
     float *scores_out;
+    /* Which tiled kernel serves the call, for A/B measurements and tests: 0 = the library chooses (by shape),
+     * 1 = the 4-wave kernel (128 query rows per work-group), 2 = the 8-wave ping-pong kernel (256 rows; needs d == 128
+     * in whole 16-byte rows and more than 128 query rows, and is ignored otherwise).  Any other value: FLASH_EINVAL.
+     * The reference selects its kernel by template flags alone (src/main.cu:141-178) and has no such switch. */
+    int kernel_hint;
+    /* Optional debug output: when non-NULL, every work-group of the tiled kernel stores FLASH_STAMP_WORDS 64-bit words
+     * at stage_stamps_out + FLASH_STAMP_WORDS * blockIdx (buffer size: flash_stage_stamps_bytes): words 0..6 are readings
+     * of the constant 100 MHz device counter -- 0 entry, 1 all prologue requests issued, 2 own requests landed,
+     * 3 first work-group barrier passed, 4 first score tile computed, 5 key-tile loop finished, 6 results stored --
+     * and word 7 packs (tiles of the work-group) << 32 | hardware id of the CU (bits 0-15 of HW_ID; bits 16-19 the
+     * XCC).  The call then runs instrumented instances of the same kernels (same arithmetic, same results).  With a
+     * split count above 1 the combine step is not stamped.  The only instrumentation of the reference is the event
+     * pair around its launches (src/main.cu:195-213). */
+    uint64_t *stage_stamps_out;
 } flash_params;
+
+#define FLASH_STAMP_WORDS 8
 
 /* Tiled forward over the whole key range: replaces
  *     forward_kernel<...><<<dim3(Tr,H,B),256,smem>>>(param)              (src/flash_forward.h:13-15, src/main.cu:189)
@@ -108,6 +124,11 @@ int flash_splitkv_workspace_bytes(const flash_params *p, size_t *o_partial_bytes
 
 /* The split count flash_forward_splitkv will use for p (after the heuristic and clamping). */
 int flash_splitkv_resolve_splits(const flash_params *p);
+
+/* Bytes of the buffer stage_stamps_out must point to for p under the given entry point (split != 0: as launched by
+ * flash_forward_splitkv, else by flash_forward): FLASH_STAMP_WORDS * 8 bytes per work-group of the tiled kernel that
+ * the call launches; 0 when the call would not run a tiled kernel (Nq == 1 decode stream, empty problem). */
+int flash_stage_stamps_bytes(const flash_params *p, int split, size_t *bytes);
 
 /* num_splits_heuristic (src/main.cu:391-422), same arguments and return value; main() passes num_SMs = 108,
  * this library's callers pass the CU count (256). */

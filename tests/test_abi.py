@@ -88,6 +88,10 @@ def test_argument_errors_are_codes_not_aborts(fa):
         assert entry(C.byref(_params(fa, H=6, H_kv=4)), None) == E_INVAL  # query heads must be a multiple of K/V heads
         assert entry(C.byref(_params(fa, H=2, H_kv=4)), None) == E_INVAL
         assert entry(C.byref(_params(fa, H=2, H_kv=-1)), None) == E_INVAL
+        assert entry(C.byref(_params(fa, kernel_hint=3)), None) == E_INVAL
+        assert entry(C.byref(_params(fa, kernel_hint=-1)), None) == E_INVAL
+        assert entry(C.byref(_params(fa, stage_stamps_out=0x6004)), None) == E_ALIGN
+        assert entry(C.byref(_params(fa, Nq=2 ** 30, Nk=2 ** 30, d=1)), None) == E_INVAL
         # empty problems are a no-op
         assert entry(C.byref(_params(fa, B=0)), None) == 0
         assert entry(C.byref(_params(fa, Nq=0, Q=None, O=None, LSE=None)), None) == 0
@@ -133,6 +137,34 @@ def test_split_resolution_and_workspace(fa):
     assert fa.resolve_splits(1, 1, 1, 300, 64, 0) == 1
     with pytest.raises(fa.FlashError):
         fa.resolve_splits(1, 1, 1, 128, 64, 1000)
+
+
+def test_stage_stamp_buffer_size(fa):
+    L = fa.lib()
+    nb = C.c_size_t(99)
+    words = 8 * fa.FLASH_STAMP_WORDS
+    # causal prefill benchmark shape: 8-wave kernel, 256 rows per work-group; 128 with the 4-wave kernel
+    p = _params(fa, B=4, H=16, Nq=2048, Nk=2048, d=128, is_causal=1)
+    assert L.flash_stage_stamps_bytes(C.byref(p), 0, C.byref(nb)) == 0 and nb.value == 64 * 8 * words
+    p.kernel_hint = 1
+    assert L.flash_stage_stamps_bytes(C.byref(p), 0, C.byref(nb)) == 0 and nb.value == 64 * 16 * words
+    # split entry point: one row per work-group of the split launch; the decode stream is not stamped
+    p = _params(fa, B=1, H=4, Nq=1021, Nk=1021, d=31, num_splits=3)
+    assert L.flash_stage_stamps_bytes(C.byref(p), 1, C.byref(nb)) == 0 and nb.value == 4 * 8 * 3 * words
+    p = _params(fa, B=16, H=32, Nq=1, Nk=16384, d=128, num_splits=16)
+    assert L.flash_stage_stamps_bytes(C.byref(p), 1, C.byref(nb)) == 0 and nb.value == 0
+    # eight query heads per K/V head decoding together: heads become rows of the tiled kernel
+    p = _params(fa, B=16, H=32, H_kv=4, Nq=1, Nk=16384, d=128, num_splits=16)
+    assert L.flash_stage_stamps_bytes(C.byref(p), 1, C.byref(nb)) == 0 and nb.value == 16 * 4 * 16 * words
+    assert L.flash_stage_stamps_bytes(C.byref(_params(fa, B=0)), 0, C.byref(nb)) == 0 and nb.value == 0
+    assert L.flash_stage_stamps_bytes(C.byref(p), 1, None) == E_INVAL
+
+
+def test_no_environment_lookups_in_the_dispatch():
+    csrc = os.path.join(ROOT, "flash_attn_amd", "csrc")
+    for f in os.listdir(csrc):
+        if f.endswith((".hip", ".h")):
+            assert "getenv" not in open(os.path.join(csrc, f)).read(), f
 
 
 def test_dropout_threshold_matches_oracle(fa, oracle):

@@ -185,6 +185,8 @@ def test_grouped_query_heads(fa, oracle, H, Hk, Nq, Nk, d, kw):
     (32, 1, 64, 1111, dict()),                        # 32 per group
     (8, 2, 72, 900, dict()),                          # head dim not a bucket width
     (12, 2, 31, 700, dict()),                         # 6 per group, odd head dim
+    (32, 2, 128, 2500, dict(window=(-1, 0))),         # "causal" written as a right window of 0: must not cut a head's keys
+    (32, 2, 128, 2500, dict(window=(-1, 3))),
 ])
 def test_grouped_query_decode(fa, oracle, H, Hk, d, Nk, kw):
     B = 2
@@ -201,6 +203,79 @@ def test_grouped_query_decode(fa, oracle, H, Hk, d, Nk, kw):
     for S in (1, 6):
         o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=S, **gkw)
         check_o_lse(o, lse, O, L, f"GQA decode H={H} Hk={Hk} S={S}")
+
+
+# One query row under grouped heads: the three routes of the split entry point (heads as rows of the tiled kernel,
+# streaming kernel with G heads per work-group, tiled fallback) each see every mask family.
+@pytest.mark.parametrize("G", [1, 3, 4, 8, 16])
+@pytest.mark.parametrize("window", [(-1, -1), (-1, 0), (-1, 5), (700, 0), (700, -1)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_decode_routes_times_masks(fa, oracle, G, window, causal):
+    B, Hk, d, Nk = 2, 2, 128, 1300
+    H = Hk * G
+    q = randn_f16_gpu((B, H, 1, d), 41)
+    k = randn_f16_gpu((B, Hk, Nk, d), 42)
+    v = randn_f16_gpu((B, Hk, Nk, d), 43)
+    kr, vr = (t.repeat_interleave(G, dim=1).contiguous() for t in (k, v))
+    O, L = oracle_forward_batched(oracle, q, kr, vr, window=window, causal=causal)
+    for extra in (dict(), dict(dropout_p=0.0, softmax_scale=d ** -0.5)):
+        o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=4, window=window, causal=causal, **extra)
+        check_o_lse(o, lse, O, L, f"decode G={G} window={window} causal={causal}")
+    # the element-wise tiled fallback (odd head dim) under the same masks
+    q2, k2, v2 = q[..., :31].contiguous(), k[..., :31].contiguous(), v[..., :31].contiguous()
+    O2, L2 = oracle_forward_batched(oracle, q2, k2.repeat_interleave(G, dim=1), v2.repeat_interleave(G, dim=1),
+                                    window=window, causal=causal)
+    o, lse = fa.flash_forward_splitkv(q2, k2, v2, num_splits=3, window=window, causal=causal)
+    check_o_lse(o, lse, O2, L2, f"decode odd d G={G} window={window} causal={causal}")
+
+
+def test_unbounded_windows_written_as_large_numbers(fa):
+    """A window bound that cannot cut (INT_MAX is a common spelling of "off") equals no bound, bit for bit."""
+    import torch
+    big = 2 ** 31 - 1
+    q, k, v = _qkv(1, 2, 300, 333, 64, seed=3)
+    for causal in (False, True):
+        o0, l0 = fa.flash_forward(q, k, v, causal=causal)
+        for w in ((big, big), (big, -1), (-1, big), (333, 300), (10 ** 9, 5)):
+            ref = (o0, l0) if w[1] != 5 else fa.flash_forward(q, k, v, causal=causal, window=(-1, 5))
+            o, l = fa.flash_forward(q, k, v, causal=causal, window=w)
+            assert torch.equal(o, ref[0]) and torch.equal(l, ref[1]), (w, causal)
+    q1 = q[:, :, :1].contiguous()
+    o0, l0 = fa.flash_forward_splitkv(q1, k, v, num_splits=2)
+    o, l = fa.flash_forward_splitkv(q1, k, v, num_splits=2, window=(big, big))
+    assert torch.equal(o, o0) and torch.equal(l, l0)
+
+
+@pytest.mark.parametrize("hint,N,d,kw", [
+    (2, 600, 128, dict(causal=True)),                 # 8-wave kernel
+    (1, 600, 128, dict(causal=True)),                 # 4-wave kernel, tiles fetched straight into LDS
+    (0, 300, 64, dict(window=(100, 0))),              # 4-wave kernel, register-staged tiles
+    (0, 150, 31, dict()),                             # element-wise instance
+])
+def test_stage_stamps(fa, oracle, hint, N, d, kw):
+    """Debug output: per work-group stamps of the constant 100 MHz counter are non-decreasing from stage to stage, the
+    last word carries the tile count, and the instrumented instance returns what the plain one returns."""
+    import torch
+    B, H = 2, 3
+    q, k, v = _qkv(B, H, N, N, d, seed=hint + N)
+    o0, l0 = fa.flash_forward(q, k, v, kernel_hint=hint, **kw)
+    o, l, st = fa.flash_forward(q, k, v, kernel_hint=hint, return_stage_stamps=True, **kw)
+    assert torch.equal(o, o0) and torch.equal(l, l0)
+    O, L = oracle_forward_batched(oracle, q, k, v, **kw)
+    check_o_lse(o, l, O, L, "instrumented instance")
+    rows = 256 if hint == 2 else 128
+    assert st.shape == (B * H * ((N + rows - 1) // rows), fa.FLASH_STAMP_WORDS)
+    t = st.cpu().numpy()
+    assert (t[:, 0] > 0).all()
+    assert (np.diff(t[:, :7], axis=1) >= 0).all(), "stamps must not run backwards"
+    assert ((t[:, 6] - t[:, 0]) < 100_000_000).all()  # less than a second
+    tiles = t[:, 7] >> 32
+    assert tiles.min() >= 1 and tiles.max() <= (N + 63) // 64
+    # split entry point: one stamp row per work-group of the split launch
+    o, l, st2 = fa.flash_forward_splitkv(q, k, v, num_splits=2, kernel_hint=hint, return_stage_stamps=True, **kw)
+    check_o_lse(o, l, O, L, "instrumented split instance")
+    assert st2.shape[0] == 2 * st.shape[0]
+    assert (np.diff(st2.cpu().numpy()[:, :7], axis=1) >= 0).all()
 
 
 def test_grouped_query_head_counts_must_divide(fa):
@@ -262,7 +337,7 @@ def test_full_size_properties_decode(fa):
     assert torch.allclose(o.float(), torch.full_like(o, 0.5, dtype=torch.float32), atol=1e-3)
 
 
-# The 8-wave kernel (d = 128; by preference only large grids of long rows, forced here through FLASH_ATTN_KERNEL):
+# The 8-wave kernel (d = 128; by preference only large grids of long rows, forced here through kernel_hint):
 # ragged lengths, Nq != Nk in both directions, every mask incl. narrow windows, grouped heads, dropout, split mode.
 @pytest.mark.parametrize("Nq,Nk,Hk,kw", [
     (1100, 1100, 2, dict(causal=True)),
@@ -277,15 +352,14 @@ def test_full_size_properties_decode(fa):
     (513, 700, 2, dict(window=(40, 3))),
     (129, 129, 2, dict()),
 ])
-def test_eight_wave_kernel_cases(fa, oracle, Nq, Nk, Hk, kw, monkeypatch):
+def test_eight_wave_kernel_cases(fa, oracle, Nq, Nk, Hk, kw):
     import torch
-    monkeypatch.setenv("FLASH_ATTN_KERNEL", "8wave")
     B, H, d = 1, 2, 128
     q = randn_f16_gpu((B, H, Nq, d), 21)
     k = randn_f16_gpu((B, Hk, Nk, d), 22)
     v = randn_f16_gpu((B, Hk, Nk, d), 23)
     kr, vr = (t.repeat_interleave(H // Hk, dim=1).contiguous() for t in (k, v))
-    kw = dict(kw)
+    kw = dict(kw, kernel_hint=fa.KERNEL_8WAVE)
     okw = {x: kw[x] for x in ("causal", "window") if x in kw}
     if kw.pop("alibi", False):
         sl, sl_t = _slopes(oracle, H)
