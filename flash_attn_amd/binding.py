@@ -15,6 +15,7 @@ FLASH_OK = 0
 FLASH_MAX_HEAD_DIM = 128
 FLASH_MAX_SPLITS = 128
 FLASH_STAMP_WORDS = 8
+FLASH_STATIC_SCRATCH_BYTES = 32 << 20
 KERNEL_AUTO, KERNEL_4WAVE, KERNEL_8WAVE = 0, 1, 2
 
 
@@ -73,6 +74,8 @@ def lib():
         L.flash_forward.argtypes = [pp, C.c_void_p]
         L.flash_forward_splitkv.restype = C.c_int
         L.flash_forward_splitkv.argtypes = [pp, C.c_void_p]
+        L.flash_forward_splitkv_static.restype = C.c_int
+        L.flash_forward_splitkv_static.argtypes = [pp, C.c_void_p]
         L.flash_splitkv_workspace_bytes.restype = C.c_int
         L.flash_splitkv_workspace_bytes.argtypes = [pp, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
         L.flash_splitkv_resolve_splits.restype = C.c_int

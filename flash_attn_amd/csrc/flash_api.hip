@@ -190,6 +190,31 @@ int resolve_splits(const flash_params* p)
     return s;
 }
 
+// ---- built-in split workspace of flash_forward_splitkv_static (for callers that cannot allocate).
+// A file-scope device array: every GPU the library runs on holds its own copy, at its own address, until the process
+// ends.  In host code the array's name only stands for the symbol; the device address comes from hipGetSymbolAddress,
+// looked up once per device with that device current, and only that address is ever handed to a kernel.
+constexpr size_t kScratchBytes = FLASH_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+int scratch_of_current_device(unsigned char** out)
+{
+    static std::atomic<unsigned char*> addr[fa::kMaxDevices];
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return record_hip((int)e);
+    if (dev < 0 || dev >= fa::kMaxDevices) return FLASH_ENODEVICE;
+    unsigned char* p = addr[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        void* sym = nullptr;
+        if (hipError_t e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)); e != hipSuccess) return record_hip((int)e);
+        if (sym == nullptr) return FLASH_ENODEVICE;
+        p = static_cast<unsigned char*>(sym);
+        addr[dev].store(p, std::memory_order_release);  // (a concurrent first call stores the same address)
+    }
+    *out = p;
+    return FLASH_OK;
+}
+
 // Which kernel serves a split-KV call; may reshape the arguments (grouped decode).
 constexpr int kRouteTiled = 0, kRouteStream = 1;
 int splitkv_route(const flash_params* p, fa::FwdArgs* a)
@@ -215,6 +240,20 @@ int splitkv_route(const flash_params* p, fa::FwdArgs* a)
     return kRouteTiled;
 }
 
+// split kernel (+ combine) for an already validated p and its resolved split count
+int run_splitkv(const flash_params* p, int splits, hipStream_t st)
+{
+    if (splits > 1 && (!p->O_partial || !p->LSE_partial)) return FLASH_EWORKSPACE;
+    if (splits > 1 && (misaligned(p->O_partial, 16) || misaligned(p->LSE_partial, 4))) return FLASH_EALIGN;
+    if (const int rc = device_usable(); rc != FLASH_OK) return rc;
+    fa::FwdArgs a;
+    fill_args(p, splits, &a);
+    const int route = splitkv_route(p, &a);
+    const int e = route == kRouteStream ? record_hip(fa::launch_decode_split(a, st)) : launch_tiled(p, a, st);
+    if (e != FLASH_OK || splits == 1) return e;
+    return record_hip(fa::launch_combine(a, st));
+}
+
 }  // namespace
 
 #define FLASH_EXPORT __attribute__((visibility("default")))
@@ -235,19 +274,33 @@ FLASH_EXPORT int flash_forward(const flash_params* p, void* stream)
 FLASH_EXPORT int flash_forward_splitkv(const flash_params* p, void* stream)
 {
     bool empty;
+    const int rc = validate(p, &empty);
+    if (rc != FLASH_OK || empty) return rc;
+    return run_splitkv(p, resolve_splits(p), static_cast<hipStream_t>(stream));
+}
+
+FLASH_EXPORT int flash_forward_splitkv_static(const flash_params* p, void* stream)
+{
+    bool empty;
     int rc = validate(p, &empty);
     if (rc != FLASH_OK || empty) return rc;
     const int splits = resolve_splits(p);
-    if (splits > 1 && (!p->O_partial || !p->LSE_partial)) return FLASH_EWORKSPACE;
-    if (splits > 1 && (misaligned(p->O_partial, 16) || misaligned(p->LSE_partial, 4))) return FLASH_EALIGN;
-    if ((rc = device_usable()) != FLASH_OK) return rc;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    fa::FwdArgs a;
-    fill_args(p, splits, &a);
-    const int route = splitkv_route(p, &a);
-    const int e = route == kRouteStream ? record_hip(fa::launch_decode_split(a, st)) : launch_tiled(p, a, st);
-    if (e != FLASH_OK || splits == 1) return e;
-    return record_hip(fa::launch_combine(a, st));
+    flash_params q = *p;
+    q.O_partial = nullptr;
+    q.LSE_partial = nullptr;
+    if (splits > 1) {
+        // O_partial at the start of the scratch array, LSE_partial behind it on the next 256-byte boundary.  Every
+        // element the combine step reads is written by the split kernel of the same call, so nothing is cleared.
+        const size_t rows = (size_t)p->B * p->H * splits * p->Nq;
+        const size_t o_bytes = (rows * p->d * sizeof(float) + 255) & ~(size_t)255;
+        if (o_bytes + rows * sizeof(float) > kScratchBytes) return FLASH_ESCRATCH;
+        if ((rc = device_usable()) != FLASH_OK) return rc;
+        unsigned char* base = nullptr;
+        if ((rc = scratch_of_current_device(&base)) != FLASH_OK) return rc;
+        q.O_partial = reinterpret_cast<float*>(base);
+        q.LSE_partial = reinterpret_cast<float*>(base + o_bytes);
+    }
+    return run_splitkv(&q, splits, static_cast<hipStream_t>(stream));
 }
 
 FLASH_EXPORT int flash_stage_stamps_bytes(const flash_params* p, int split, size_t* bytes)
@@ -342,6 +395,7 @@ FLASH_EXPORT const char* flash_strerror(int code)
         case FLASH_ESPLITS: return "too many splits";
         case FLASH_ELAUNCH: return "HIP launch failed";
         case FLASH_ENODEVICE: return "the current device is not a gfx950";
+        case FLASH_ESCRATCH: return "split workspace exceeds the built-in scratch (FLASH_STATIC_SCRATCH_BYTES)";
         default: return "unknown error";
     }
 }

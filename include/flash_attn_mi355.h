@@ -28,7 +28,8 @@ enum {
     FLASH_EWORKSPACE = -4,   /* num_splits > 1 but O_partial / LSE_partial missing                           */
     FLASH_ESPLITS = -5,      /* num_splits larger than FLASH_MAX_SPLITS                                      */
     FLASH_ELAUNCH = -6,      /* the HIP runtime rejected a launch; see flash_last_hip_error()                */
-    FLASH_ENODEVICE = -7     /* the current device is not a gfx950 (the library carries code for nothing else) */
+    FLASH_ENODEVICE = -7,    /* the current device is not a gfx950 (the library carries code for nothing else) */
+    FLASH_ESCRATCH = -8      /* flash_forward_splitkv_static: the split workspace would not fit the built-in scratch */
 };
 
 #define FLASH_MAX_HEAD_DIM 128
@@ -118,6 +119,20 @@ int flash_forward(const flash_params *p, void *stream);
  * which streams K and V once and is bound by memory bandwidth, enough splits of at least 512 keys to give every CU
  * several work-groups.  flash_splitkv_resolve_splits returns the count either way. */
 int flash_forward_splitkv(const flash_params *p, void *stream);
+
+/* flash_forward_splitkv for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose main() allocates O_tmp, L and M
+ * itself (src/main.cu:160-162).  Same arguments, same kernels and bit-identical results, but O_partial / LSE_partial of
+ * p are ignored: the split partials go to a scratch array built into the library's device code, FLASH_STATIC_SCRATCH_BYTES
+ * per GPU, held from the moment the library is loaded on that GPU until the process ends.  The call allocates and
+ * frees nothing.  Its first call on a device looks up the array's address there (hipGetSymbolAddress) and, like every
+ * entry point, the first launch of a kernel instance raises that kernel's dynamic-LDS limit: make one ordinary call
+ * per device and shape class before capturing.  A problem whose partials need more than the scratch
+ * (flash_splitkv_workspace_bytes: both sizes, the first rounded up to 256) returns FLASH_ESCRATCH and launches nothing.
+ * All calls on one GPU share the array: calls that may overlap on that GPU (different streams, different threads)
+ * race on it and must be serialised by the caller, or use flash_forward_splitkv with workspaces of their own. */
+#define FLASH_STATIC_SCRATCH_BYTES (32u << 20)
+int flash_forward_splitkv_static(const flash_params *p, void *stream);
 
 /* Bytes of O_partial and of LSE_partial needed for p (the cudaMallocs of src/main.cu:160-162). Either may be NULL. */
 int flash_splitkv_workspace_bytes(const flash_params *p, size_t *o_partial_bytes, size_t *lse_partial_bytes);

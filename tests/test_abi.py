@@ -99,7 +99,13 @@ def test_argument_errors_are_codes_not_aborts(fa):
     assert L.flash_forward_splitkv(C.byref(_params(fa, Nk=1024, num_splits=4)), None) == E_WORKSPACE
     # odd head dims only need element alignment
     assert L.flash_forward(C.byref(_params(fa, d=31, Q=0x1001)), None) == E_ALIGN
-    for code in (0, -1, -2, -3, -4, -5, -6, -7):
+    # the entry point that brings its own scratch: same checks, and a size limit instead of the workspace check
+    assert L.flash_forward_splitkv_static(None, None) == E_INVAL
+    assert L.flash_forward_splitkv_static(C.byref(_params(fa, d=129)), None) == E_HEADDIM
+    assert L.flash_forward_splitkv_static(C.byref(_params(fa, B=0)), None) == 0
+    big = _params(fa, B=64, H=64, Nq=1, Nk=16384, d=128, num_splits=128)  # 270 MB of partials
+    assert L.flash_forward_splitkv_static(C.byref(big), None) == -8
+    for code in (0, -1, -2, -3, -4, -5, -6, -7, -8):
         assert L.flash_strerror(code)
     assert b"head_dim" in L.flash_strerror(E_HEADDIM)
 
