@@ -164,6 +164,40 @@ def time_steps(step, steps, warmup):
     return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
 
 
+def stage_timeline(fa, c, q, k, v):
+    """Per-work-group time stamps of the instrumented kernel instance (flash_params.stage_stamps_out, a debug output of
+    the library): where a work-group of this workload spends its time, in microseconds of the 100 MHz device counter."""
+    import numpy as np
+    import torch
+
+    slopes = None
+    if c["alibi"]:
+        slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / c["H"]) for h in range(c["H"])], dtype=torch.float32, device="cuda")
+    kw = dict(causal=c["causal"], window=c["window"], alibi_slopes=slopes, dropout_p=c["p"], seed=1234, offset=0)
+    for _ in range(3):
+        fa.flash_forward(q, k, v, **kw)
+    torch.cuda.synchronize()
+    st = fa.flash_forward(q, k, v, return_stage_stamps=True, **kw)[-1]
+    torch.cuda.synchronize()
+    t = st.cpu().numpy().astype(np.int64)
+    t0 = t[:, 0].min()
+    names = fa.stage_stamp_names()
+    rel = (t[:, 1:7] - t[:, :1]) / 100.0
+    tiles = t[:, 7] >> 32
+    loop = (t[:, 5] - t[:, 4]) / 100.0
+    out = {"work_groups": int(t.shape[0]), "first_entry_to_last_exit_us": float((t[:, 6].max() - t0) / 100.0),
+           "mean_lifetime_us": float(rel[:, 5].mean()),
+           "us_after_entry": {names[i + 1]: {"mean": float(rel[:, i].mean()), "min": float(rel[:, i].min()),
+                                             "max": float(rel[:, i].max())} for i in range(6)},
+           "tiles_per_group": {"mean": float(tiles.mean()), "max": int(tiles.max())},
+           "us_per_tile_in_loop": float(loop.sum() / max(1, int((tiles - 1).clip(min=0).sum()))),
+           "epilogue_us": float((rel[:, 5] - rel[:, 4]).mean())}
+    xcc = (t[:, 7] >> 16) & 0xf
+    cu_se = (t[:, 7] & 0xffff) >> 8  # CU, SH and SE fields of HW_ID
+    out["distinct_cus"] = int(len(set(zip(xcc.tolist(), cu_se.tolist()))))
+    return out
+
+
 def mfma_sustained():
     """Sustained 32x32x16 fp16 MFMA rate of this GPU for zero / constant / random operands, measured by the stand-alone
     probe tests/driver/mfma_rate (a child process; a fraction of a second).  None when the probe is not built."""
@@ -232,6 +266,8 @@ def main():
     ap.add_argument("--cpu-slices", type=int, default=16)
     ap.add_argument("--steady-launches", type=int, default=1000,
                     help="launches of the steady-state leg (the reference times 1000, src/main.cu:187-213); 0 = skip")
+    ap.add_argument("--stage-timeline", action="store_true",
+                    help="print the per-stage timeline of the headline workload (instrumented kernel instance) and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain elementwise kernel reading and writing 256 MiB each, so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled against a known transfer")
@@ -258,6 +294,9 @@ def main():
     name = args.workload
     c = CONFIGS[name] if name in CONFIGS else DIAG[name]
     q, k, v = make_inputs(c)
+    if args.stage_timeline:
+        print(json.dumps({"workload": f"{name}: {DESCR[name]}", "stage_timeline": stage_timeline(fa, c, q, k, v)}))
+        return
     step, _ = make_step(fa, c, q, k, v)
     host_ms, ev_ms = time_steps(step, args.steps, args.warmup)
     if c["Nq"] == 1:
