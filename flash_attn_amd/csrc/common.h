@@ -47,6 +47,7 @@ struct FwdArgs {
     int keys_per_split;  // multiple of 128
     int Tr;              // number of query row blocks
     int kernel_hint;     // 0: by shape, 1: 4-wave kernel, 2: 8-wave kernel where it can serve the call
+    int alibi_left;      // ALiBi and no visible key lies right of its row (causal, or right window 0)
 
     // index of the K/V slice [Nk,d] read by query slice bh = b * H + h
     __device__ __forceinline__ int kv_slice(int bh) const { return (bh / H) * Hk + (bh % H) / kv_group; }
@@ -107,6 +108,13 @@ struct Stamps {
     }
 };
 
+// two fp32 -> packed fp16, round to nearest even, in one instruction (v_cvt_pk_f16_f32)
+__device__ __forceinline__ v2h pack_f16(float a, float b)
+{
+    const v2f t = {a, b};
+    return __builtin_convertvector(t, v2h);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
@@ -128,6 +136,9 @@ __device__ __forceinline__ void mul_wide_u32(uint32_t m, uint32_t x, uint32_t& h
     lo = (uint32_t)r;
 }
 
+// three-input exclusive or in one instruction (v_bitop3_b32, truth table 0x96)
+__device__ __forceinline__ uint32_t xor3(uint32_t a, uint32_t b, uint32_t c) { return __builtin_amdgcn_bitop3_b32(a, b, c, 0x96); }
+
 __device__ __forceinline__ v4u philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1)
 {
 #pragma unroll
@@ -135,9 +146,9 @@ __device__ __forceinline__ v4u philox4x32_10(uint32_t c0, uint32_t c1, uint32_t 
         uint32_t hi0, lo0, hi1, lo1;
         mul_wide_u32(0xD2511F53u, c0, hi0, lo0);
         mul_wide_u32(0xCD9E8D57u, c2, hi1, lo1);
-        c0 = hi1 ^ c1 ^ k0;
+        c0 = xor3(hi1, c1, k0);
         c1 = lo1;
-        c2 = hi0 ^ c3 ^ k1;
+        c2 = xor3(hi0, c3, k1);
         c3 = lo0;
         k0 += 0x9E3779B9u;
         k1 += 0xBB67AE85u;

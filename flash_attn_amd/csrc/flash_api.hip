@@ -115,6 +115,7 @@ void fill_args(const flash_params* p, int splits, fa::FwdArgs* a)
     // as no bound; callers write "unbounded" as INT_MAX too, which the kernels' i' + right would overflow.
     a->wl = p->window_left >= p->Nk ? -1 : p->window_left;
     a->wr = p->window_right >= p->Nq ? -1 : p->window_right;
+    a->alibi_left = (p->alibi_slopes && (a->causal || a->wr == 0)) ? 1 : 0;
     a->scale_log2 = p->softmax_scale * fa::kLog2e;
     a->drop_thr = flash_dropout_threshold(p->dropout_p);
     a->drop_rscale = 1.0f / (1.0f - p->dropout_p);

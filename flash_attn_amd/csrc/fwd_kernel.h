@@ -23,6 +23,8 @@
 //    reference zero-fills them and leaves them unmasked).  Head dims that are not a multiple of 8 use the
 //    element-wise load / store path (kVec = false).
 #pragma once
+#include <type_traits>
+
 #include "common.h"
 
 namespace fa {
@@ -91,7 +93,9 @@ __device__ __forceinline__ v4u load_chunk(const half_t* __restrict__ rowp, int c
 constexpr float kLazyTau = 8.0f;
 
 // variant bits of the kernel template
-constexpr int kVarVec = 1, kVarAlibi = 2, kVarDropout = 4, kVarFullD = 8, kVarStamp = 16;  // kVarStamp: debug time stamps
+// kVarStamp: debug time stamps.  kVarAlibiLeft (with kVarAlibi, kVarVec): every visible key lies at or left of its row
+// (causal mask or a right window of 0), which lets the bias ride in the MFMA accumulator (see calib below).
+constexpr int kVarVec = 1, kVarAlibi = 2, kVarDropout = 4, kVarFullD = 8, kVarStamp = 16, kVarAlibiLeft = 32;
 
 template <int D, int NB, int VAR>
 __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 0 ? 3 : 2) : 1) fwd_kernel(const FwdArgs a)
@@ -102,7 +106,9 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     Stamps<kStamp> stamps;
     stamps.take(0);
     constexpr int BC = C::BC, KS = C::KS, MB = C::MB, CH = C::CH, SK = C::SK, SV = C::SV, NLD = C::NLD;
-    constexpr bool kDma = C::DMA && kVec && kFullD && (D >= 128 || !kDropout);
+    // (the folded-ALiBi instances also take the direct path at small head dims: the sixteen bias constants need the
+    // registers that the staged loads would occupy)
+    constexpr bool kDma = kVec && kFullD && ((C::DMA && (D >= 128 || !kDropout)) || (VAR & kVarAlibiLeft) != 0);
     constexpr int NSTG = kDma ? C::NSTG : 2;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     char* const Ks = smem;
@@ -307,6 +313,17 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
         nsig = scale_late ? -slope2 / c2 : 0.0f;
     }
 
+    // ALiBi where every visible key lies at or left of its row (causal mask, or a right window of 0: j <= i, keys right
+    // of the row are masked anyway): |i - j| = i - j splits into a part that only depends on the accumulator register,
+    // -nsig * (8 (r / 4) + r % 4), and a part per lane and 32-key block.  The first goes into the MFMA as the initial
+    // accumulator value, the second into the addend of the exponent fma: no instruction per score is left.
+    constexpr bool kFoldAlibi = kAlibi && kVec && (VAR & kVarAlibiLeft) != 0;
+    v16f calib;
+    if constexpr (kFoldAlibi) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) calib[r] = -nsig * (float)(8 * (r >> 2) + (r & 3));
+    }
+
     // LDS read offsets of this lane
     const int k_rd = l32 * SK + g * 16;                                          // + kb*32*SK + ks*32
     const int v_rd = (4 * g + ((lane & 15) >> 2)) * SV + (((lane >> 4) & 1) * 16 + (lane & 3) * 4) * 2;  // + row/col blocks
@@ -314,12 +331,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
 
     // S^T = K Q^T of the tile in K buffer `buf`
     auto qk = [&](int buf, v16f (&s)[2][NB]) {
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) s[kb][nb][r] = 0.0f;
+        constexpr bool folded = kFoldAlibi;
         const char* kbase = Ks + buf * C::KBUF + k_rd;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
@@ -327,8 +339,22 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
             for (int kb = 0; kb < 2; ++kb) {
                 const v8h af = *reinterpret_cast<const v8h*>(kbase + kb * 32 * SK + ks * 32);
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
-                    s[kb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, qf[nb][ks], s[kb][nb], 0, 0, 0);
+                for (int nb = 0; nb < NB; ++nb) {
+                    if (ks == 0) {
+                        // first k-step: the accumulator starts from zero (an inline constant) or, with the ALiBi bias
+                        // folded in, from the per-register bias constants, which stay where they are
+                        if constexpr (folded) {
+                            // written out: the compiler only knows the form whose result overwrites the addend and would
+                            // copy the sixteen constants for every tile
+                            asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(s[kb][nb]) : "v"(af), "v"(qf[nb][ks]), "v"(calib));
+                        } else {
+                            const v16f z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                            s[kb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, qf[nb][ks], z, 0, 0, 0);
+                        }
+                    } else {
+                        s[kb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, qf[nb][ks], s[kb][nb], 0, 0, 0);
+                    }
+                }
             }
         }
         // issue order: kQkAhead fragment reads first, then read and MFMA in turn (left to itself the compiler waits
@@ -349,9 +375,16 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     // mask_sides: bit 0 = some row of the wave has its first allowed key inside or after this tile, bit 1 = some row
     // has its last allowed key inside or before it (both wave-uniform)
     auto softmax = [&](int mask_sides, int kb0, v16f (&s)[2][NB], v8h (&pf)[2][2][NB]) {
+        constexpr bool folded = kFoldAlibi;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-            if constexpr (kAlibi) {
+            // folded ALiBi: bias of 32-key block kb that is common to the lane's 16 scores there (score units)
+            float abias[2] = {0.0f, 0.0f};
+            if constexpr (folded) {
+                abias[0] = nsig * (iif[nb] - (float)(kb0 + 4 * g));
+                abias[1] = abias[0] - nsig * 32.0f;
+            }
+            if constexpr (kAlibi && !folded) {
                 // score*scale - slope*|i - j|  (src/main.cu:315,324), in the log2 domain
                 const float jb = (float)(kb0 + 4 * g) - iif[nb];
                 if (scale_late) {
@@ -410,10 +443,19 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                 }
             }
             float mx = -INFINITY;
+            if constexpr (folded) {
+                float mk[2] = {-INFINITY, -INFINITY};
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+                for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kb][nb][r]);
+                    for (int r = 0; r < 16; ++r) mk[kb] = fmaxf(mk[kb], s[kb][nb][r]);
+                mx = fmaxf(mk[0] + abias[0], mk[1] + abias[1]);
+            } else {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kb][nb][r]);
+            }
             mx = xhalf_max(mx);
             mx *= cs;  // cs > 0
             if (__builtin_amdgcn_ballot_w64(mx > m_ref[nb] + kLazyTau) != 0ull) {
@@ -430,13 +472,15 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
             const float m_use = (m_ref[nb] == -INFINITY) ? 0.0f : m_ref[nb];  // nothing seen yet: exp2(-inf - 0) = 0
             float rs = 0.0f;
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int kb = 0; kb < 2; ++kb) {
+                const float addend = folded ? __builtin_fmaf(abias[kb], cs, -m_use) : -m_use;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const float p = fast_exp2(__builtin_fmaf(s[kb][nb][r], cs, -m_use));
+                    const float p = fast_exp2(__builtin_fmaf(s[kb][nb][r], cs, addend));
                     rs += p;
                     s[kb][nb][r] = p;
                 }
+            }
             l_run[nb] += rs;  // per-lane partial; the two half-waves are added in the epilogue
             if constexpr (kDropout) {
                 // drop iff field < threshold, row sum left undropped (src/flash_forward.h:221-237); the survivors' factor
@@ -469,7 +513,11 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
 #pragma unroll
                 for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) pf[kb][tt][nb][e] = (half_t)s[kb][nb][8 * tt + e];
+                    for (int e = 0; e < 8; e += 2) {
+                        const v2h h2 = pack_f16(s[kb][nb][8 * tt + e], s[kb][nb][8 * tt + e + 1]);
+                        pf[kb][tt][nb][e] = h2[0];
+                        pf[kb][tt][nb][e + 1] = h2[1];
+                    }
         }
     };
 
@@ -516,8 +564,8 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
         if (wave_live && kb0 <= hi_max && kb0 + BC - 1 >= lo_min) {
             v16f s[2][NB];
             v8h pf[2][2][NB];
-            qk(buf, s);
             const int mask_sides = (kb0 < lo_max ? 1 : 0) | (kb0 + BC - 1 > hi_min ? 2 : 0);
+            qk(buf, s);
             softmax(mask_sides, kb0, s, pf);
             pv(buf, pf);
         }
@@ -689,26 +737,29 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
     return launch_kernel(kern, dim3((unsigned)groups), dim3(256), smem, st, a);
 }
 
-// The nine instances of a bucket: {d == bucket, d % 8 == 0} x {plain, ALiBi, dropout, both}, and the element-wise
-// path with both features compiled in (slope 0 / threshold 0 make them identities, so it serves every request
+// The instances of a bucket: {d == bucket, d % 8 == 0} x {plain, ALiBi, ALiBi with every visible key at or left of its
+// row, dropout, both}, and the element-wise path with both features compiled in (slope 0 / threshold 0 make them identities, so it serves every request
 // with d % 8 != 0).  ST = kVarStamp selects their instrumented twins (debug time stamps).
 template <int D, int NB, int ST>
 inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
 {
     hipError_t e;
     const int feat = variant & (kVarAlibi | kVarDropout);
+    constexpr int AL = kVarAlibi | kVarAlibiLeft;  // ALiBi with no visible key right of its row
     if (!(variant & kVarVec)) {
         e = launch_fwd_instance<D, NB, ST | kVarAlibi | kVarDropout>(a, st);
     } else if (a.d == D) {
-        if (feat == 0) e = launch_fwd_instance<D, NB, ST | kVarVec | kVarFullD>(a, st);
-        else if (feat == kVarAlibi) e = launch_fwd_instance<D, NB, ST | kVarVec | kVarFullD | kVarAlibi>(a, st);
-        else if (feat == kVarDropout) e = launch_fwd_instance<D, NB, ST | kVarVec | kVarFullD | kVarDropout>(a, st);
-        else e = launch_fwd_instance<D, NB, ST | kVarVec | kVarFullD | kVarAlibi | kVarDropout>(a, st);
+        constexpr int V = ST | kVarVec | kVarFullD;
+        if (feat == 0) e = launch_fwd_instance<D, NB, V>(a, st);
+        else if (feat == kVarAlibi) e = a.alibi_left ? launch_fwd_instance<D, NB, V | AL>(a, st) : launch_fwd_instance<D, NB, V | kVarAlibi>(a, st);
+        else if (feat == kVarDropout) e = launch_fwd_instance<D, NB, V | kVarDropout>(a, st);
+        else e = a.alibi_left ? launch_fwd_instance<D, NB, V | AL | kVarDropout>(a, st) : launch_fwd_instance<D, NB, V | kVarAlibi | kVarDropout>(a, st);
     } else {
-        if (feat == 0) e = launch_fwd_instance<D, NB, ST | kVarVec>(a, st);
-        else if (feat == kVarAlibi) e = launch_fwd_instance<D, NB, ST | kVarVec | kVarAlibi>(a, st);
-        else if (feat == kVarDropout) e = launch_fwd_instance<D, NB, ST | kVarVec | kVarDropout>(a, st);
-        else e = launch_fwd_instance<D, NB, ST | kVarVec | kVarAlibi | kVarDropout>(a, st);
+        constexpr int V = ST | kVarVec;
+        if (feat == 0) e = launch_fwd_instance<D, NB, V>(a, st);
+        else if (feat == kVarAlibi) e = a.alibi_left ? launch_fwd_instance<D, NB, V | AL>(a, st) : launch_fwd_instance<D, NB, V | kVarAlibi>(a, st);
+        else if (feat == kVarDropout) e = launch_fwd_instance<D, NB, V | kVarDropout>(a, st);
+        else e = a.alibi_left ? launch_fwd_instance<D, NB, V | AL | kVarDropout>(a, st) : launch_fwd_instance<D, NB, V | kVarAlibi | kVarDropout>(a, st);
     }
     return (int)e;
 }

@@ -415,7 +415,11 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-                for (int e = 0; e < 8; ++e) pf[kb][tt][e] = (half_t)s[kb][8 * tt + e];
+                for (int e = 0; e < 8; e += 2) {
+                    const v2h h2 = pack_f16(s[kb][8 * tt + e], s[kb][8 * tt + e + 1]);
+                    pf[kb][tt][e] = h2[0];
+                    pf[kb][tt][e + 1] = h2[1];
+                }
     };
 
     // One iteration.  The four stage pointers are distinct LDS regions; declaring them restrict is what lets the
