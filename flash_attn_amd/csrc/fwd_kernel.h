@@ -307,11 +307,9 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     const float c2 = a.scale_log2;
     const bool scale_late = kVec || c2 > 0.0f;
     const float cs = scale_late ? c2 : 1.0f;
+    // The ALiBi slope of the head is read once the first tile requests are on their way (read_slope below): it is a
+    // vector load, the wait for it counts every older request as well, and nothing before the first softmax needs it.
     float slope2 = 0.0f, nsig = 0.0f;
-    if constexpr (kAlibi) {
-        slope2 = a.alibi ? a.alibi[h] * kLog2e : 0.0f;
-        nsig = scale_late ? -slope2 / c2 : 0.0f;
-    }
 
     // ALiBi where every visible key lies at or left of its row (causal mask, or a right window of 0: j <= i, keys right
     // of the row are masked anyway): |i - j| = i - j splits into a part that only depends on the accumulator register,
@@ -319,10 +317,17 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     // accumulator value, the second into the addend of the exponent fma: no instruction per score is left.
     constexpr bool kFoldAlibi = kAlibi && kVec && (VAR & kVarAlibiLeft) != 0;
     v16f calib;
-    if constexpr (kFoldAlibi) {
+    auto read_slope = [&]() {
+        if constexpr (kAlibi) {
+            // (the vector instances are only launched with a slope table; the element-wise one serves every request)
+            slope2 = (kVec || a.alibi) ? a.alibi[h] * kLog2e : 0.0f;
+            nsig = scale_late ? -slope2 / c2 : 0.0f;
+            if constexpr (kFoldAlibi) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) calib[r] = -nsig * (float)(8 * (r >> 2) + (r & 3));
-    }
+                for (int r = 0; r < 16; ++r) calib[r] = -nsig * (float)(8 * (r >> 2) + (r & 3));
+            }
+        }
+    };
 
     // LDS read offsets of this lane
     const int k_rd = l32 * SK + g * 16;                                          // + kb*32*SK + ks*32
@@ -579,6 +584,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
 #pragma unroll
         for (int u = 0; u < PF; ++u)
             if (u < ntiles) dma_tile(tile_begin + u, u);
+        read_slope();
         stamps.take(1);
         dma_wait(PF == 2 && ntiles > 1);
         pin_q();
@@ -601,6 +607,9 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
         if (ntiles > 0) {
             gload(Kbh, tile_begin, kreg);
             gload(Vbh, tile_begin, vreg);
+        }
+        read_slope();
+        if (ntiles > 0) {
             stamps.take(1);
             put_k(0);
             put_v(0);

@@ -209,8 +209,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     // into the exponent (one fma per score): cs = scale, and the ALiBi bias is added beforehand divided by the scale.
     // (The host sends a non-positive scale to the element-wise instance of the 4-wave kernel.)
     const float c2 = a.scale_log2, cs = c2;
-    float nsig = 0.0f;
-    if constexpr (kAlibi) nsig = a.alibi ? -(a.alibi[h] * kLog2e) / c2 : 0.0f;
+    float nsig = 0.0f;  // ALiBi slope / scale, negated: read behind the prologue requests (below)
 
     // Lane parts of the fragment addresses (layout above).  K fragment (ks, kb): key 32 kb + l32, chunk 2 ks + g
     // -> k_rd ^ (32 ks) + 8192 kb.  V transpose read (st, mb, half h) of lane (G = lane / 16, e = lane / 4 % 4,
@@ -474,6 +473,8 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
             }
             if (ntiles > 2) load_k(2, Ks + 2 * C::KBUF);
         }
+        // (a vector load: the wait for it counts every older request too, so it goes last; only launched with a table)
+        if constexpr (kAlibi) nsig = -(a.alibi[h] * kLog2e) / c2;
         stamps.take(1);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (a memory clobber: the reads below stay below)
         stamps.take(2);
