@@ -183,24 +183,58 @@ __global__ void __launch_bounds__(256) decode_split_kernel(const FwdArgs a)
     }
 }
 
+// Reductions over the 64 lanes of a wave without LDS: DPP inside the rows of 16 lanes, v_permlane32_swap between the
+// halves, v_readlane for the last two rows; the result is wave-uniform.
+__device__ __forceinline__ float wave_sum(float v)
+{
+    v = xhalf_sum(group_sum<16>(v));  // lanes of rows r and r ^ 2 now hold the total of both rows
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0)) +
+           __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+}
+__device__ __forceinline__ float wave_max(float v)
+{
+    v = fmaxf(v, dpp_mov<0xB1>(v));
+    v = fmaxf(v, dpp_mov<0x4E>(v));
+    v = fmaxf(v, dpp_mov<0x141>(v));
+    v = fmaxf(v, dpp_mov<0x140>(v));
+    v = xhalf_max(v);
+    return fmaxf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0)),
+                 __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16)));
+}
+
 // One wave per query row: LSE = logsumexp_s LSE_s, O = sum_s exp(LSE_s - LSE) O_s
 // (same value as m = max M_s, l = sum e^{M_s-m} L_s, O = sum (L_s e^{M_s-m} / l) O_s of splitkv.h:359-397).
+// The weights of a row live in LDS that only its wave touches, so no work-group barrier is needed.  With d % 8 == 0
+// a lane holds four consecutive columns, the two halves of the wave take the even and the odd splits, and the first
+// partial rows are requested before the log-sum-exp values they will be weighted with.
 __global__ void __launch_bounds__(256) combine_kernel(const float* __restrict__ O_partial,
                                                       const float* __restrict__ LSE_partial, half_t* __restrict__ O,
                                                       float* __restrict__ LSE, int BH, int Nq, int d, int S)
 {
     __shared__ float s_w[4][FLASH_MAX_SPLITS_K];
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = wave_uniform(threadIdx.x >> 6);
     const long long row = (long long)blockIdx.x * 4 + wave;
-    const long long rows = (long long)BH * Nq;
-    const bool valid = row < rows;
-    const int bh = valid ? (int)(row / Nq) : 0, i = valid ? (int)(row % Nq) : 0;
+    if (row >= (long long)BH * Nq) return;
+    const int bh = (int)(row / Nq), i = (int)(row % Nq);
     const float* lp = LSE_partial + (size_t)bh * S * Nq + i;  // stride Nq between splits
+    const size_t sstride = (size_t)Nq * d;                     // floats between the partial rows of two splits
+    const float* op = O_partial + ((size_t)bh * S * Nq + i) * d;
+    const bool vec = (d & 7) == 0;  // rows of the partials and of O are 16-byte aligned (the host checks the bases)
+    constexpr int U = 4;            // partial rows in flight per half-wave
+    const int c4 = (lane & 31) * 4, grp = lane >> 5;
+    const bool act = c4 < d;
+    float4 pre[U];
+    if (vec) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int s = grp + 2 * u;
+            pre[u] = (act && s < S) ? *reinterpret_cast<const float4*>(op + s * sstride + c4) : float4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
     float mx = -INFINITY;
     for (int s = lane; s < S; s += 64) mx = fmaxf(mx, lp[(size_t)s * Nq]);
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    mx = wave_max(mx);
     const float mu = (mx == -INFINITY) ? 0.0f : mx;
     float sum = 0.0f;
     for (int s = lane; s < S; s += 64) {
@@ -208,17 +242,38 @@ __global__ void __launch_bounds__(256) combine_kernel(const float* __restrict__ 
         s_w[wave][s] = w;
         sum += w;
     }
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o, 64);
+    sum = wave_sum(sum);
     const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
-    __syncthreads();
-    if (!valid) return;
-    for (int dc = lane; dc < d; dc += 64) {
-        float o = 0.0f;
-        for (int s = 0; s < S; ++s) o += s_w[wave][s] * O_partial[(((size_t)bh * S + s) * Nq + i) * d + dc];
-        O[((size_t)bh * Nq + i) * d + dc] = (half_t)(o * inv);
-    }
     if (lane == 0) LSE[(size_t)bh * Nq + i] = sum > 0.0f ? mx + __logf(sum) : -INFINITY;
+    if (vec) {
+        float4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int s = grp + 2 * u;
+            const float w = s < S ? s_w[wave][s] : 0.0f;
+            acc.x += w * pre[u].x, acc.y += w * pre[u].y, acc.z += w * pre[u].z, acc.w += w * pre[u].w;
+        }
+        if (act) {
+            for (int s = grp + 2 * U; s < S; s += 2) {
+                const float4 o = *reinterpret_cast<const float4*>(op + s * sstride + c4);
+                const float w = s_w[wave][s];
+                acc.x += w * o.x, acc.y += w * o.y, acc.z += w * o.z, acc.w += w * o.w;
+            }
+        }
+        acc.x = xhalf_sum(acc.x), acc.y = xhalf_sum(acc.y), acc.z = xhalf_sum(acc.z), acc.w = xhalf_sum(acc.w);
+        if (act && grp == 0) {
+            union { v2h h[2]; uint2 u; } r;
+            r.h[0] = pack_f16(acc.x * inv, acc.y * inv);
+            r.h[1] = pack_f16(acc.z * inv, acc.w * inv);
+            *reinterpret_cast<uint2*>(O + ((size_t)bh * Nq + i) * d + c4) = r.u;
+        }
+    } else {
+        for (int dc = lane; dc < d; dc += 64) {
+            float o = 0.0f;
+            for (int s = 0; s < S; ++s) o += s_w[wave][s] * op[s * sstride + dc];
+            O[((size_t)bh * Nq + i) * d + dc] = (half_t)(o * inv);
+        }
+    }
 }
 
 // keep[b,h,i,j] = (16-bit field dropout_field(j) of the Philox call dropout_call(j) of row (b*H + h, i)) >= threshold;
