@@ -199,8 +199,9 @@ def stage_timeline(fa, c, q, k, v):
 
 
 def mfma_sustained():
-    """Sustained 32x32x16 fp16 MFMA rate of this GPU for zero / constant / random operands, measured by the stand-alone
-    probe tests/driver/mfma_rate (a child process; a fraction of a second).  None when the probe is not built."""
+    """Sustained 32x32x16 fp16 MFMA rate of this GPU for zero / constant / random operands, and for random operands
+    with the companion instructions of an attention loop beside every MFMA, measured by the stand-alone probe
+    tests/driver/mfma_rate (a child process; about a second).  None when the probe is not built."""
     exe = os.path.join(ROOT, "tests", "driver", "mfma_rate")
     if not os.path.exists(exe):
         return None
@@ -325,6 +326,9 @@ def main():
         if sus:
             roof["mfma_sustained"] = sus
             roof["frac_of_sustained_random"] = roof["achieved"] / sus["random"]
+            if sus.get("random_attention_mix"):
+                # MFMAs on random operands with one LDS fragment read, four fma and one exp issued beside each
+                roof["frac_of_attention_mix_ceiling"] = roof["achieved"] / sus["random_attention_mix"]
 
     result = {
         "metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -3,7 +3,13 @@
 // MFMA pipe is the only busy unit.  The rate depends on the data: with changing, random operands the power management
 // of the MI355X lowers the clock well below what zero or constant operands run at, so the number printed for "random"
 // is the ceiling a real attention kernel can approach, whatever its schedule.
-// Prints one JSON line: {"zeros": T, "constant": T, "random": T} in TFLOP/s (best of 5 launches each).
+// A fourth figure, "random_attention_mix", is the rate of the same MFMAs on random operands when every MFMA is
+// accompanied by what an attention loop at head dim 128 with 32 query rows per wave has to issue beside it: one
+// re-read of an A fragment from LDS (half of them ds_read_b128 as for K, half pairs of ds_read_b64_tr_b16 as for V),
+// four fp32 fma/add and one v_exp_f32 -- all independent of each other and of the MFMAs, 8 waves per CU, no global
+// memory traffic, no barriers, no masks: the ceiling of that instruction mix, whatever the schedule.
+// Prints one JSON line: {"zeros": T, "constant": T, "random": T, "random_attention_mix": T} in TFLOP/s (best of 5
+// launches each).
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
@@ -60,6 +66,89 @@ __global__ void __launch_bounds__(256) mfma_loop(float* out, int iters)
     out[blockIdx.x * blockDim.x + threadIdx.x] = r_;
 }
 
+// The MFMA stream of mfma_loop<2> with the companions of an attention loop (see the head of the file).  One work-group of
+// 8 waves per CU; 64 KiB of LDS hold four stages of random fp16 data that the fragment reads walk through.
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef __fp16 v4hp __attribute__((__vector_size__(4 * sizeof(__fp16))));
+#define LDS_AS __attribute__((address_space(3)))
+__global__ void __launch_bounds__(512) attention_mix_loop(float* out, int iters)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    LDS_AS char* lds = (LDS_AS char*)smem;
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    unsigned s = tid * 2654435761u + blockIdx.x * 40503u + 12345u;
+    auto rnd2 = [&]() {  // two fp16 values of magnitude 0.125 .. 2 with random sign and mantissa
+        auto h = [](unsigned x) { return (x & 0x8000u) | ((12u + ((x >> 10) & 3u)) << 10) | (x & 0x3ffu); };
+        s = s * 1664525u + 1013904223u;
+        const unsigned lo = s >> 16;
+        s = s * 1664525u + 1013904223u;
+        return h(lo) | (h(s >> 16) << 16);
+    };
+    for (int i = tid; i < 16384; i += 512) ((LDS_AS unsigned*)lds)[i] = rnd2();
+    __syncthreads();
+    // lane parts of conflict-free fragment addresses in a row-major 64 x 128 fp16 tile with permuted 16-byte chunks
+    const int k_rd = l32 * 256 + ((g ^ (l32 & 1)) << 4) + (((l32 & 15) >> 1) << 5);
+    const int G = lane >> 4, e4 = (lane >> 2) & 3, j4 = lane & 3;
+    const int v_rd = (4 * (G >> 1) + e4) * 256 + (((G & 1) ^ (G >> 1)) << 5) + 8 * j4 + (e4 << 6);
+    union Frag { v4u u; v8h h; v4hp p[2]; };
+    Frag fr[16], bq;
+    for (int i = 0; i < 16; ++i) fr[i].u = v4u{rnd2(), rnd2(), rnd2(), rnd2()};
+    bq.u = v4u{rnd2(), rnd2(), rnd2(), rnd2()};
+    v16f acc[4];
+    for (int n = 0; n < 4; ++n)
+        for (int r = 0; r < 16; ++r) acc[n][r] = 0.f;
+    float vr[8];
+    for (int i = 0; i < 8; ++i) vr[i] = tid * 1e-3f + i;
+    const float c1 = 0.999f, c0 = 0.01f;
+    for (int it = 0; it < iters; ++it) {
+        unsigned kb = (unsigned)k_rd + (it & 3) * 16384, vb = (unsigned)v_rd + (it & 3) * 16384;
+        asm volatile("" : "+v"(kb), "+v"(vb));
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            // the fragment consumed here was requested one iteration ago; its refill is issued right behind the MFMA
+            acc[u & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fr[u].h, bq.h, acc[u & 3], 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(vr[(u * 4 + v) & 7]) : "v"(c1), "v"(c0));
+            asm volatile("v_exp_f32 %0, %0" : "+v"(vr[(u + 3) & 7]));
+            if (u < 8) {
+                fr[u].u = *(LDS_AS const v4u*)(lds + (kb ^ (unsigned)((u & 7) << 5)) + (u >> 3) * 8192);
+            } else {
+                LDS_AS char* p = lds + (vb ^ (unsigned)((u & 3) << 6)) + (u >> 2) * 4096;
+                fr[u].p[0] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((LDS_AS v4hp*)p);
+                fr[u].p[1] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((LDS_AS v4hp*)(p + 2048));
+            }
+        }
+    }
+    float r_ = 0;
+    for (int n = 0; n < 4; ++n)
+        for (int r = 0; r < 16; ++r) r_ += acc[n][r];
+    for (int i = 0; i < 8; ++i) r_ += vr[i];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = r_;
+}
+
+double best_mix_tflops(float* out, int n_cu)
+{
+    const int iters = 12000, lds_bytes = 65536;
+    HIP_CHECK(hipFuncSetAttribute((const void*)attention_mix_loop, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
+    hipLaunchKernelGGL(attention_mix_loop, n_cu, 512, lds_bytes, 0, out, 10);
+    HIP_CHECK(hipDeviceSynchronize());
+    hipEvent_t e0, e1;
+    HIP_CHECK(hipEventCreate(&e0));
+    HIP_CHECK(hipEventCreate(&e1));
+    double best = 0;
+    for (int rep = 0; rep < 5; ++rep) {
+        HIP_CHECK(hipEventRecord(e0, 0));
+        hipLaunchKernelGGL(attention_mix_loop, n_cu, 512, lds_bytes, 0, out, iters);
+        HIP_CHECK(hipEventRecord(e1, 0));
+        HIP_CHECK(hipEventSynchronize(e1));
+        float ms;
+        HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+        const double t = (double)n_cu * 8 * iters * 16 * 32768.0 / ms / 1e9;
+        if (t > best) best = t;
+    }
+    return best;
+}
+
 template <typename K>
 double best_tflops(K kern, float* out, int n_cu)
 {
@@ -94,7 +183,9 @@ int main()
     const double z = best_tflops(mfma_loop<0>, out, n_cu);
     const double c = best_tflops(mfma_loop<1>, out, n_cu);
     const double r = best_tflops(mfma_loop<2>, out, n_cu);
-    std::printf("{\"zeros\": %.1f, \"constant\": %.1f, \"random\": %.1f, \"unit\": \"TFLOP/s\", \"cus\": %d}\n", z, c, r, n_cu);
+    const double m = best_mix_tflops(out, n_cu);
+    std::printf("{\"zeros\": %.1f, \"constant\": %.1f, \"random\": %.1f, \"random_attention_mix\": %.1f, \"unit\": \"TFLOP/s\", \"cus\": %d}\n",
+                z, c, r, m, n_cu);
     HIP_CHECK(hipFree(out));
     return 0;
 }
