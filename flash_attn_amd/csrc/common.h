@@ -136,6 +136,58 @@ __device__ __forceinline__ void mul_wide_u32(uint32_t m, uint32_t x, uint32_t& h
     lo = (uint32_t)r;
 }
 
+// Element masks of a 32 x 32 score block whose boundary runs along its diagonal.  In the accumulator layout lane
+// (l32 = lane % 32, g = lane / 32) holds in register r the score of query row l32 and key 8 (r / 4) + r % 4 + 4 g of the
+// block, so "key right of the diagonal" (key > row) and "key left of it" (key < row) are fixed sets of lanes per register:
+// sixteen 64-bit constants each, applied with one v_cndmask per register on a constant lane mask instead of a comparison
+// and a select per score.
+constexpr uint64_t diag_lane_mask(int r, bool right)
+{
+    uint64_t m = 0;
+    for (int lane = 0; lane < 64; ++lane) {
+        const int row = lane & 31, key = 8 * (r >> 2) + (r & 3) + 4 * (lane >> 5);
+        if (right ? key > row : key < row) m |= 1ull << lane;
+    }
+    return m;
+}
+template <bool kRight, int R = 0>
+__device__ __forceinline__ void mask_off_diagonal(v16f& s, float ninf)
+{
+    if constexpr (R < 16) {
+        // (the constant goes into vcc inside the statement: as an operand the compiler would keep all thirty-two
+        // constants in scalar registers across the key loop and spill them)
+        constexpr uint64_t m = diag_lane_mask(R, kRight);
+        asm("s_mov_b32 vcc_lo, %2\n\ts_mov_b32 vcc_hi, %3\n\tv_cndmask_b32_e32 %0, %0, %1, vcc"
+            : "+v"(s[R])
+            : "v"(ninf), "n"((uint32_t)m), "n"((uint32_t)(m >> 32))
+            : "vcc");
+        mask_off_diagonal<kRight, R + 1>(s, ninf);
+    }
+}
+
+// The general case: the score in register R belongs to key 8 (R / 4) + R % 4 of the block (the caller folds the lane's
+// 4 g and the block's position into the bound); scores of keys above (below) the lane's bound become -inf.  In place
+// and as inline asm on purpose: written as selects the compiler copies the sixteen accumulator registers first, and
+// turns a rare wave-uniform branch around them into selects that every tile executes.
+template <bool kAbove, int R = 0>
+__device__ __forceinline__ void mask_beyond(v16f& s, int bound, float ninf)
+{
+    if constexpr (R < 16) {
+        constexpr int key = 8 * (R >> 2) + (R & 3);
+        if constexpr (kAbove)
+            asm("v_cmp_gt_i32_e32 vcc, %2, %1\n\tv_cndmask_b32_e32 %0, %0, %3, vcc" : "+v"(s[R]) : "v"(bound), "n"(key), "v"(ninf) : "vcc");
+        else
+            asm("v_cmp_lt_i32_e32 vcc, %2, %1\n\tv_cndmask_b32_e32 %0, %0, %3, vcc" : "+v"(s[R]) : "v"(bound), "n"(key), "v"(ninf) : "vcc");
+        mask_beyond<kAbove, R + 1>(s, bound, ninf);
+    }
+}
+
+__device__ __forceinline__ void mask_whole_block(v16f& s, float ninf)
+{
+#pragma unroll
+    for (int r = 0; r < 16; ++r) asm("v_mov_b32 %0, %1" : "=v"(s[r]) : "v"(ninf));
+}
+
 // three-input exclusive or in one instruction (v_bitop3_b32, truth table 0x96)
 __device__ __forceinline__ uint32_t xor3(uint32_t a, uint32_t b, uint32_t c) { return __builtin_amdgcn_bitop3_b32(a, b, c, 0x96); }
 

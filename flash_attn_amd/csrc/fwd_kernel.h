@@ -407,31 +407,34 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                 }
             }
             if (mask_sides != 0) {
-                // Wave-uniform and rare (boundary tiles only).  Routing the bounds through an empty volatile asm keeps
-                // these real branches: otherwise the compiler folds the blocks into selects that every tile executes.
-                // A tile that only one end of the interval crosses takes one comparison per score.
-                int lo_rel = lo[nb] - kb0 - 4 * g, hi_rel = hi[nb] - kb0 - 4 * g;
-                asm volatile("; boundary tile: element mask" : "+v"(lo_rel), "+v"(hi_rel));
-                if (mask_sides == 1) {
+                // Wave-uniform and rare (boundary tiles only); the masking itself is inline asm (common.h), which keeps
+                // these real branches.  The bounds of the wave's rows run along block diagonals when they move by one
+                // key per row and start at a multiple of 32 (causal masks and windows whose offsets are multiples of 32,
+                // rows not clipped by a sequence or split end): then lane-mask constants per 32-key block do the
+                // masking; otherwise a tile takes one comparison per score and crossed end of the interval.
+                const float ninf = -INFINITY;
+                const bool hi_diag = NB == 1 && hi_max - hi_min == 31 && (hi_min & 31) == 0;
+                const bool lo_diag = NB == 1 && lo_max - lo_min == 31 && (lo_min & 31) == 0;
+                if (((mask_sides & 1) == 0 || lo_diag) && ((mask_sides & 2) == 0 || hi_diag)) {
 #pragma unroll
-                    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r)
-                            if (32 * kb + 8 * (r >> 2) + (r & 3) < lo_rel) s[kb][nb][r] = -INFINITY;
-                } else if (mask_sides == 2) {
-#pragma unroll
-                    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r)
-                            if (32 * kb + 8 * (r >> 2) + (r & 3) > hi_rel) s[kb][nb][r] = -INFINITY;
-                } else {
-#pragma unroll
-                    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            const int jr = 32 * kb + 8 * (r >> 2) + (r & 3);
-                            if (jr < lo_rel || jr > hi_rel) s[kb][nb][r] = -INFINITY;
+                    for (int kb = 0; kb < 2; ++kb) {
+                        // last / first visible key of the wave's first row relative to the block: multiples of 32
+                        const int dh = (mask_sides & 2) ? hi_min - (kb0 + 32 * kb) : 64;
+                        const int dl = (mask_sides & 1) ? lo_min - (kb0 + 32 * kb) : -64;
+                        if (dh < 0 || dl >= 32) {
+                            mask_whole_block(s[kb][nb], ninf);
+                        } else {
+                            if (dh == 0) mask_off_diagonal<true>(s[kb][nb], ninf);
+                            if (dl == 0) mask_off_diagonal<false>(s[kb][nb], ninf);
                         }
+                    }
+                } else {
+                    const int lo_rel = lo[nb] - kb0 - 4 * g, hi_rel = hi[nb] - kb0 - 4 * g;
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb) {
+                        if (mask_sides & 1) mask_beyond<false>(s[kb][nb], lo_rel - 32 * kb, ninf);
+                        if (mask_sides & 2) mask_beyond<true>(s[kb][nb], hi_rel - 32 * kb, ninf);
+                    }
                 }
             }
             if constexpr (!kVec) {

@@ -331,29 +331,36 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
                     s[kb][r] = __builtin_fmaf(nsig, __builtin_fabsf(jb + (float)(32 * kb + 8 * (r >> 2) + (r & 3))), s[kb][r]);
         }
         if (mask_sides != 0) {
-            // a tile that only one end of the interval crosses takes one comparison per score
-            int lo_rel = lo - kb0 - 4 * g, hi_rel = hi - kb0 - 4 * g;
-            asm volatile("; boundary tile: element mask" : "+v"(lo_rel), "+v"(hi_rel));
-            if (mask_sides == 1) {
+            // Wave-uniform and rare (boundary tiles only); the masking itself is inline asm (common.h), which keeps these
+            // real branches.  Where the bounds of the wave's rows run along block diagonals (one key per row, from a
+            // multiple of 32: causal masks and windows whose offsets are multiples of 32, rows not clipped by a sequence
+            // or split end), lane-mask constants per 32-key block do the masking; otherwise a tile takes one
+            // comparison per score and crossed end of the interval.
+            const float ninf = -INFINITY;
+            const int hi_f = __builtin_amdgcn_readlane(hi, 0), hi_l = __builtin_amdgcn_readlane(hi, 31);
+            const int lo_f = __builtin_amdgcn_readlane(lo, 0), lo_l = __builtin_amdgcn_readlane(lo, 31);
+            const bool hi_diag = hi_l - hi_f == 31 && (hi_f & 31) == 0;
+            const bool lo_diag = lo_l - lo_f == 31 && (lo_f & 31) == 0;
+            if (((mask_sides & 1) == 0 || lo_diag) && ((mask_sides & 2) == 0 || hi_diag)) {
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        if (32 * kb + 8 * (r >> 2) + (r & 3) < lo_rel) s[kb][r] = -INFINITY;
-            } else if (mask_sides == 2) {
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        if (32 * kb + 8 * (r >> 2) + (r & 3) > hi_rel) s[kb][r] = -INFINITY;
-            } else {
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int jr = 32 * kb + 8 * (r >> 2) + (r & 3);
-                        if (jr < lo_rel || jr > hi_rel) s[kb][r] = -INFINITY;
+                for (int kb = 0; kb < 2; ++kb) {
+                    // last / first visible key of the wave's first row relative to the block: multiples of 32
+                    const int dh = (mask_sides & 2) ? hi_f - (kb0 + 32 * kb) : 64;
+                    const int dl = (mask_sides & 1) ? lo_f - (kb0 + 32 * kb) : -64;
+                    if (dh < 0 || dl >= 32) {
+                        mask_whole_block(s[kb], ninf);
+                    } else {
+                        if (dh == 0) mask_off_diagonal<true>(s[kb], ninf);
+                        if (dl == 0) mask_off_diagonal<false>(s[kb], ninf);
                     }
+                }
+            } else {
+                const int lo_rel = lo - kb0 - 4 * g, hi_rel = hi - kb0 - 4 * g;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+                    if (mask_sides & 1) mask_beyond<false>(s[kb], lo_rel - 32 * kb, ninf);
+                    if (mask_sides & 2) mask_beyond<true>(s[kb], hi_rel - 32 * kb, ninf);
+                }
             }
         }
         float mx = -INFINITY;

@@ -57,6 +57,25 @@ def test_nq_differs_from_nk(fa, oracle, Nq, Nk):
         check_o_lse(o, lse, O, L, f"Nq={Nq} Nk={Nk} {list(kw)}")
 
 
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("Nq,Nk", [(520, 520), (480, 544), (500, 520), (96, 544)])
+def test_mask_bounds_along_block_diagonals(fa, oracle, Nq, Nk, d):
+    """Causal masks and windows whose offsets are multiples of 32 put the bounds of a wave's 32 rows on the diagonals of
+    32 x 32 score blocks, which the kernels mask with lane-mask constants; ragged ends, a shift Nk - Nq that is no
+    multiple of 32 and split boundaries send the same requests down the per-score comparison instead."""
+    q, k, v = _qkv(1, 2, Nq, Nk, d, seed=23)
+    for window in ((0, 0), (32, 0), (0, 32), (32, 32), (64, 96), (256, 0), (-1, 0), (-1, 64), (96, -1)):
+        for causal in (False, True):
+            O, L = oracle_forward_batched(oracle, q, k, v, window=window, causal=causal)
+            o, lse = fa.flash_forward(q, k, v, window=window, causal=causal)
+            check_o_lse(o, lse, O, L, f"Nq={Nq} Nk={Nk} d={d} window={window} causal={causal}")
+            o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=3, window=window, causal=causal)
+            check_o_lse(o, lse, O, L, f"3 splits Nq={Nq} Nk={Nk} d={d} window={window} causal={causal}")
+            if d == 128 and Nq > 128:
+                o, lse = fa.flash_forward(q, k, v, window=window, causal=causal, kernel_hint=fa.KERNEL_8WAVE)
+                check_o_lse(o, lse, O, L, f"8-wave Nq={Nq} Nk={Nk} window={window} causal={causal}")
+
+
 @pytest.mark.parametrize("window", [(0, 0), (1, 0), (0, 3), (100, 100), (128, 128), (256, 0), (5, 300), (-1, 7), (9, -1)])
 def test_windows(fa, oracle, window):
     """window (128,128) is the reference's own window_attention setting (src/main.cu:57-60)."""
