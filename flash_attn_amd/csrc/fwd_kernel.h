@@ -50,10 +50,6 @@ struct FwdCfg {
     static constexpr int KBUF = BC * SK;
     static constexpr int VBUF = BC * SV;
     static constexpr int SMEM = 2 * KBUF + 2 * VBUF;
-    // At D >= 96 the instances whose rows are whole 16-byte chunks of exactly D columns fetch their tiles straight into
-    // LDS (global_load_lds_dwordx4) instead of through registers (measured: +6-12 % at D = 128, +3-7 % at D = 96
-    // without dropout, -2.5 % with it, within +-2 % at D = 64).
-    static constexpr bool DMA = D >= 96;
     static constexpr int NSTG = 2;
     static constexpr int SMEM_DMA = NSTG * (KBUF + VBUF);
     static constexpr int NKX = (CH + 1 + 3) / 4;  // 1 KiB blocks of a K tile (CH + 1 of them) per wave, rounded up
@@ -106,9 +102,9 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     Stamps<kStamp> stamps;
     stamps.take(0);
     constexpr int BC = C::BC, KS = C::KS, MB = C::MB, CH = C::CH, SK = C::SK, SV = C::SV, NLD = C::NLD;
-    // (the folded-ALiBi instances also take the direct path at small head dims: the sixteen bias constants need the
-    // registers that the staged loads would occupy)
-    constexpr bool kDma = kVec && kFullD && ((C::DMA && (D >= 128 || !kDropout)) || (VAR & kVarAlibiLeft) != 0);
+    // Instances whose rows are whole 16-byte chunks of exactly D columns fetch their tiles straight into LDS
+    // (global_load_lds_dwordx4) instead of through registers: measured +6-12 % at D = 128, +1-4 % at D = 64 and 96.
+    constexpr bool kDma = kVec && kFullD;
     constexpr int NSTG = kDma ? C::NSTG : 2;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     char* const Ks = smem;
