@@ -285,42 +285,49 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         }
     };
     // MFMA phase body after the barrier: O += P V(t) with the first K(t+1) fragments fetched under its last MFMAs,
-    // then S = K(t+1) Q^T.  One basic block, so that the read / MFMA interleaving below can be pinned.  After the last
-    // tile the K stage holds stale data and the resulting S is never used (one wasted QK per row block).
-    auto mfma_phase = [&](uint32_t vbase, uint32_t kbase) {
+    // then S = K(t+1) Q^T.  One basic block, so that the read / MFMA interleaving below can be pinned.  The wave's last
+    // tile has no successor whose scores it could use: its phase (last_c true) is the PV part alone.
+    auto mfma_phase = [&](auto last_c, uint32_t vbase, uint32_t kbase) __attribute__((always_inline)) {
+        constexpr bool kLast = decltype(last_c)::value;
         pv_mfma(0);
         __builtin_amdgcn_sched_barrier(0);  // step 0 first: its fragments were requested first
         v_read(vbase, 2);
         pv_mfma(1);
         v_read(vbase, 3);
         pv_mfma(2);
+        if constexpr (!kLast) {
 #pragma unroll
-        for (int ks = 0; ks < KPD; ++ks) k_read(kbase, ks);
+            for (int ks = 0; ks < KPD; ++ks) k_read(kbase, ks);
+        }
         pv_mfma(3);
-        s_clear();
+        if constexpr (!kLast) {
+            s_clear();
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            if (ks + KPD < KS) k_read(kbase, ks + KPD);
-            qk_mfma(ks);
+            for (int ks = 0; ks < KS; ++ks) {
+                if (ks + KPD < KS) k_read(kbase, ks + KPD);
+                qk_mfma(ks);
+            }
         }
         // pin the order: [2MB reads][MB MFMA][2MB reads][MB MFMA][2*KPD reads][MB MFMA]{[2 reads][2 MFMA]}...
         __builtin_amdgcn_sched_group_barrier(0x100, 2 * MB, 0);
         __builtin_amdgcn_sched_group_barrier(0x008, MB, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 2 * MB, 0);
         __builtin_amdgcn_sched_group_barrier(0x008, MB, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 * KPD, 0);
+        if constexpr (!kLast) __builtin_amdgcn_sched_group_barrier(0x100, 2 * KPD, 0);
         __builtin_amdgcn_sched_group_barrier(0x008, MB, 0);
+        if constexpr (!kLast) {
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            if (ks + KPD < KS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            for (int ks = 0; ks < KS; ++ks) {
+                if (ks + KPD < KS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            }
         }
     };
 
     // online softmax of the tile whose scores sit in s; leaves P^T packed to fp16 in pf
     // mask_sides: bit 0 = some row of the wave has its first allowed key inside or after this tile, bit 1 = some row has
     // its last allowed key inside or before it (both wave-uniform)
-    auto softmax = [&](int mask_sides, int kb0) {
+    auto softmax = [&](int mask_sides, int kb0) __attribute__((always_inline)) {
         if constexpr (kAlibi) {
             // score*scale - slope*|i - j|  (src/main.cu:315,324), in the log2 domain
             const float jb = (float)(kb0 + 4 * g) - iif;
@@ -430,8 +437,8 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
 
     // One iteration.  The four stage pointers are distinct LDS regions; declaring them restrict is what lets the
     // compiler issue the fragment reads without first waiting (vmcnt) for the LDS-DMA writes into the other stages.
-    auto iteration = [&](FA_LDS const char* __restrict__ rdv, FA_LDS const char* __restrict__ rdk,
-                         FA_LDS char* __restrict__ wrk, FA_LDS char* __restrict__ wrv, int t) {
+    auto iteration = [&](auto last_c, FA_LDS const char* __restrict__ rdv, FA_LDS const char* __restrict__ rdk,
+                         FA_LDS char* __restrict__ wrk, FA_LDS char* __restrict__ wrv, int t) __attribute__((always_inline)) {
         const int kb0 = (tile_begin + t) * BC;
         // ---------------- VALU phase: request the tiles to come, softmax of tile t
         if (t + 3 < ntiles) load_k(t + 3, wrk);
@@ -447,7 +454,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         lds_barrier_keep<4 * MB>();
         // ---------------- MFMA phase: O += P(t) V(t), then S(t+1) = K(t+1) Q^T
         __builtin_amdgcn_s_setprio(1);
-        mfma_phase(vbase, kbase);
+        mfma_phase(last_c, vbase, kbase);
         __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of K(t+3), V(t+2) is in LDS
         lds_barrier();
@@ -524,9 +531,14 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     if (t_lo > t_hi) t_lo = t_hi;
     int t = 0;
     for (; t < t_lo; ++t) idle_iteration(t);
-    for (; t < t_hi; ++t)
-        iteration(Vs + (t % NST) * C::VBUF, Ks + ((t + 1) % NST) * C::KBUF, Ks + ((t + 3) % NST) * C::KBUF,
-                  Vs + ((t + 2) % NST) * C::VBUF, t);
+    for (; t < t_hi - 1; ++t)
+        iteration(std::false_type{}, Vs + (t % NST) * C::VBUF, Ks + ((t + 1) % NST) * C::KBUF,
+                  Ks + ((t + 3) % NST) * C::KBUF, Vs + ((t + 2) % NST) * C::VBUF, t);
+    if (t < t_hi) {  // the wave's last tile: no scores of a successor to compute
+        iteration(std::true_type{}, Vs + (t % NST) * C::VBUF, Ks + ((t + 1) % NST) * C::KBUF,
+                  Ks + ((t + 3) % NST) * C::KBUF, Vs + ((t + 2) % NST) * C::VBUF, t);
+        ++t;
+    }
     for (; t < ntiles; ++t) idle_iteration(t);
     if (grp == 0) lds_barrier();  // both groups pass the same number of barriers
     stamps.take(5);
