@@ -55,6 +55,9 @@ DIAG = {
     "diag_d64": dict(B=4, H=16, Nq=2048, Nk=2048, d=64, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=0),
     "diag_long": dict(B=1, H=16, Nq=8192, Nk=8192, d=128, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=0),
     "diag_window": dict(B=2, H=16, Nq=4096, Nk=4096, d=64, causal=False, window=(256, 0), alibi=False, p=0.0, splits=0),
+    "diag_many_slices": dict(B=16, H=32, Nq=1024, Nk=1024, d=128, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=0),
+    "diag_many_slices_d64": dict(B=8, H=32, Nq=2048, Nk=2048, d=64, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=0),
+    "diag_many_slices_long": dict(B=8, H=32, Nq=4096, Nk=4096, d=128, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=0),
     "diag_gqa_decode": dict(B=16, H=32, Hk=4, Nq=1, Nk=16384, d=128, causal=False, window=(-1, -1), alibi=False, p=0.0,
                             splits=16),
 }
@@ -67,6 +70,9 @@ DESCR = {
     "diag_noncausal": "non-causal fwd B=4 H=16 Nq=Nk=2048 d=128 (diagnostic)",
     "diag_d64": "causal fwd B=4 H=16 Nq=Nk=2048 d=64 (diagnostic)",
     "diag_long": "causal fwd B=1 H=16 Nq=Nk=8192 d=128 (diagnostic)",
+    "diag_many_slices": "causal fwd B=16 H=32 Nq=Nk=1024 d=128 (diagnostic)",
+    "diag_many_slices_d64": "causal fwd B=8 H=32 Nq=Nk=2048 d=64 (diagnostic)",
+    "diag_many_slices_long": "causal fwd B=8 H=32 Nq=Nk=4096 d=128 (diagnostic)",
     "diag_window": "local(256,0) fwd without ALiBi B=2 H=16 Nq=Nk=4096 d=64 (diagnostic)",
     "diag_gqa_decode": "split-KV decode, 8 query heads per K/V head, B=16 H=32 H_kv=4 Nq=1 Nk=16384 d=128 (diagnostic)",
 }

@@ -48,6 +48,7 @@ struct FwdArgs {
     int Tr;              // number of query row blocks
     int kernel_hint;     // 0: by shape, 1: 4-wave kernel, 2: 8-wave kernel where it can serve the call
     int alibi_left;      // ALiBi and no visible key lies right of its row (causal, or right window 0)
+    int slice_chunk;     // 4-wave kernel: head slices per chunk of the work-group order (set by its launcher)
 
     // index of the K/V slice [Nk,d] read by query slice bh = b * H + h
     __device__ __forceinline__ int kv_slice(int bh) const { return (bh / H) * Hk + (bh % H) / kv_group; }

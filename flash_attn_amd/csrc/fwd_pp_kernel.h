@@ -85,10 +85,15 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     const int l32 = lane & 31;
     const int g = lane >> 5;
 
-    const int BH = a.B * a.H;
-    const int id = blockIdx.x;
-    const int bh = id % BH;
-    const int rest = id / BH;
+    // work-group -> (head slice, split, row block) as in fwd_kernel: slices fastest inside a chunk of a.slice_chunk
+    // slices, heaviest row blocks first, chunk after chunk
+    int bh, rest;
+    {
+        const int per_chunk = a.slice_chunk * a.Tr * a.num_splits;
+        const int ch = blockIdx.x / per_chunk, w = blockIdx.x % per_chunk;
+        bh = ch * a.slice_chunk + w % a.slice_chunk;
+        rest = w / a.slice_chunk;
+    }
     const int split = rest % a.num_splits;
     const int m_block = a.Tr - 1 - rest / a.num_splits;
     const int h = bh % a.H;
@@ -608,6 +613,7 @@ inline hipError_t launch_fwd_pp_instance(const FwdArgs& a, hipStream_t st)
     FwdArgs b = a;
     b.Tr = (a.Nq + C::BR - 1) / C::BR;
     const long long groups = (long long)b.Tr * a.B * a.H * a.num_splits;
+    b.slice_chunk = slice_chunk_for(a.B * a.H, b.Tr * a.num_splits, kNumCus);  // one work-group per CU at a time
     return launch_kernel(kern, dim3((unsigned)groups), dim3(512), C::SMEM, st, b);
 }
 

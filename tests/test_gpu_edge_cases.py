@@ -57,6 +57,23 @@ def test_nq_differs_from_nk(fa, oracle, Nq, Nk):
         check_o_lse(o, lse, O, L, f"Nq={Nq} Nk={Nk} {list(kw)}")
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_many_head_slices_in_chunks(fa, oracle, causal):
+    """With far more work-groups than the GPU holds at once the kernels deal the head slices out in chunks (here 256
+    slices in two chunks of 128, in both tiled kernels): every (slice, row block) must still be served exactly once."""
+    B, H, N, d = 8, 32, 1024, 128
+    q, k, v = _qkv(B, H, N, N, d, seed=31)
+    o4, l4 = fa.flash_forward(q, k, v, causal=causal, kernel_hint=fa.KERNEL_4WAVE)
+    o8, l8 = fa.flash_forward(q, k, v, causal=causal, kernel_hint=fa.KERNEL_8WAVE)
+    assert (o4.float() - o8.float()).abs().max().item() <= 4e-3
+    assert (l4 - l8).abs().max().item() <= 2e-4
+    for b, h in ((0, 0), (3, 31), (4, 0), (7, 31), (5, 17)):  # first / last slice of each chunk and one inside
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        O, L = oracle_forward_batched(oracle, q[sl], k[sl], v[sl], causal=causal)
+        check_o_lse(o4[sl], l4[sl], O, L, f"4-wave slice ({b},{h}) causal={causal}")
+        check_o_lse(o8[sl], l8[sl], O, L, f"8-wave slice ({b},{h}) causal={causal}")
+
+
 @pytest.mark.parametrize("d", [64, 128])
 @pytest.mark.parametrize("Nq,Nk", [(520, 520), (480, 544), (500, 520), (96, 544)])
 def test_mask_bounds_along_block_diagonals(fa, oracle, Nq, Nk, d):
