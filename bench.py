@@ -204,6 +204,25 @@ def stage_timeline(fa, c, q, k, v):
     return out
 
 
+def shape_grid(fa):
+    """Forward rate over the customary grid of attention benchmarks: 16384 tokens per launch, sequence lengths
+    512 ... 16384, head dim 128 with 16 heads and 64 with 32, plain and causal.  Diagnostic only."""
+    out = {}
+    for d, H in ((128, 16), (64, 32)):
+        for causal in (False, True):
+            row = {}
+            for N in (512, 1024, 2048, 4096, 8192, 16384):
+                c = dict(B=16384 // N, H=H, Nq=N, Nk=N, d=d, causal=causal, window=(-1, -1), alibi=False, p=0.0, splits=0)
+                q, k, v = make_inputs(c)
+                step, _ = make_step(fa, c, q, k, v)
+                fl = flops_of(c)
+                _, ev_ms = time_steps(step, max(10, min(300, int(3e12 / fl))), 3)
+                row[f"N={N}"] = round(fl / (ev_ms * 1e-3) / 1e12, 1)
+                del q, k, v, step
+            out[f"d={d} H={H} {'causal' if causal else 'plain'}"] = row
+    return out
+
+
 def mfma_sustained():
     """Sustained 32x32x16 fp16 MFMA rate of this GPU for zero / constant / random operands, and for random operands
     with the companion instructions of an attention loop beside every MFMA, measured by the stand-alone probe
@@ -275,6 +294,9 @@ def main():
                     help="launches of the steady-state leg (the reference times 1000, src/main.cu:187-213); 0 = skip")
     ap.add_argument("--stage-timeline", action="store_true",
                     help="print the per-stage timeline of the headline workload (instrumented kernel instance) and exit")
+    ap.add_argument("--grid", action="store_true",
+                    help="print a table of forward rates over sequence lengths 512 ... 16384 at 16384 tokens per launch "
+                         "(d = 128 with 16 heads, d = 64 with 32; plain and causal) and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain elementwise kernel reading and writing 256 MiB each, so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled against a known transfer")
@@ -297,6 +319,10 @@ def main():
         torch.add(src, 1.0, out=dst)  # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
+
+    if args.grid:
+        print(json.dumps({"grid": shape_grid(fa), "unit": "TFLOP/s", "tokens_per_launch": 16384}))
+        return
 
     name = args.workload
     c = CONFIGS[name] if name in CONFIGS else DIAG[name]
