@@ -58,6 +58,7 @@ DIAG = {
     "diag_many_slices": dict(B=16, H=32, Nq=1024, Nk=1024, d=128, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=0),
     "diag_many_slices_d64": dict(B=8, H=32, Nq=2048, Nk=2048, d=64, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=0),
     "diag_many_slices_long": dict(B=8, H=32, Nq=4096, Nk=4096, d=128, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=0),
+    "diag_short": dict(B=32, H=32, Nq=512, Nk=512, d=64, causal=False, window=(-1, -1), alibi=False, p=0.0, splits=0),
     "diag_gqa_decode": dict(B=16, H=32, Hk=4, Nq=1, Nk=16384, d=128, causal=False, window=(-1, -1), alibi=False, p=0.0,
                             splits=16),
 }
@@ -73,6 +74,7 @@ DESCR = {
     "diag_many_slices": "causal fwd B=16 H=32 Nq=Nk=1024 d=128 (diagnostic)",
     "diag_many_slices_d64": "causal fwd B=8 H=32 Nq=Nk=2048 d=64 (diagnostic)",
     "diag_many_slices_long": "causal fwd B=8 H=32 Nq=Nk=4096 d=128 (diagnostic)",
+    "diag_short": "plain fwd B=32 H=32 Nq=Nk=512 d=64 (diagnostic)",
     "diag_window": "local(256,0) fwd without ALiBi B=2 H=16 Nq=Nk=4096 d=64 (diagnostic)",
     "diag_gqa_decode": "split-KV decode, 8 query heads per K/V head, B=16 H=32 H_kv=4 Nq=1 Nk=16384 d=128 (diagnostic)",
 }

@@ -584,15 +584,18 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     if constexpr (kDma) {
         // Tile t + PF is requested when tile t starts (its stage was read last during tile t - 1, behind a barrier);
         // before the barrier that ends tile t, the requests of tile t + 1 have landed, those of t + 2 may be in flight.
+        // Before tile 0 every stage is free: the prologue requests one tile per stage, so that the request which
+        // tile 0 would issue is already on its way (a work-group with few tiles otherwise pays the memory latency a
+        // second time at the end of its first tile).
         constexpr int PF = NSTG - 1;
         static_assert(PF == 1 || PF == 2, "prefetch distance");
         static_assert(C::NKX + C::NVX <= 15, "vmcnt immediate");
 #pragma unroll
-        for (int u = 0; u < PF; ++u)
+        for (int u = 0; u < NSTG; ++u)
             if (u < ntiles) dma_tile(tile_begin + u, u);
         read_slope();
         stamps.take(1);
-        dma_wait(PF == 2 && ntiles > 1);
+        dma_wait(false);
         pin_q();
         stamps.take(2);
         __syncthreads();
@@ -600,7 +603,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
         int buf = 0, nbuf = PF % NSTG;  // stages of tile t and of tile t + PF
         for (int t = 0; t < ntiles; ++t) {
             const bool more = t + PF < ntiles;
-            if (more) dma_tile(tile_begin + t + PF, nbuf);
+            if (more && t > 0) dma_tile(tile_begin + t + PF, nbuf);
             tile_math(t, buf);
             if (kStamp && t == 0) stamps.take(4);
             dma_wait(PF == 2 && more);
