@@ -41,6 +41,7 @@ struct FwdArgs {
     int causal, wl, wr;  // wl / wr < 0: unbounded
     float scale_log2;    // softmax_scale * log2(e)
     uint32_t drop_thr;   // keep iff 16-bit philox field >= drop_thr
+    uint32_t drop_sub2;  // drop_thr - 1 in both 16-bit halves (vector instances; they are launched with drop_thr >= 1)
     float drop_rscale;   // 1 / (1 - p)
     uint32_t seed_lo, seed_hi, off_lo;
     int num_splits;      // 1: write O/LSE; > 1: write the partial workspace
@@ -208,6 +209,60 @@ __device__ __forceinline__ v4u philox4x32_10(uint32_t c0, uint32_t c1, uint32_t 
     }
     v4u o = {c0, c1, c2, c3};
     return o;
+}
+
+// The same function for callers whose third counter word is the same in every lane (the head slice of a work-group):
+// they pass its first-round product 0xCD9E8D57 * c2 as (c2_hi, c2_lo), computed once on the scalar unit, and the first
+// round is left with one vector multiply; the exclusive-ors of uniform words fold into scalar ones as well.
+__device__ __forceinline__ v4u philox4x32_10_c2(uint32_t c0, uint32_t c1, uint32_t c2_hi, uint32_t c2_lo, uint32_t c3, uint32_t k0,
+                                                uint32_t k1)
+{
+    uint32_t hi0, lo0, hi1, lo1;
+    // round 1
+    mul_wide_u32(0xD2511F53u, c0, hi0, lo0);
+    uint32_t n0 = c1 ^ (c2_hi ^ k0);
+    const uint32_t u1 = c2_lo;  // uniform
+    uint32_t n2 = hi0 ^ (c3 ^ k1);
+    uint32_t n3 = lo0;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+    // round 2: its second word is still uniform
+    mul_wide_u32(0xD2511F53u, n0, hi0, lo0);
+    mul_wide_u32(0xCD9E8D57u, n2, hi1, lo1);
+    c0 = hi1 ^ (u1 ^ k0);
+    c1 = lo1;
+    uint32_t c2 = xor3(hi0, n3, k1);
+    c3 = lo0;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+#pragma unroll
+    for (int r = 2; r < 10; ++r) {
+        mul_wide_u32(0xD2511F53u, c0, hi0, lo0);
+        mul_wide_u32(0xCD9E8D57u, c2, hi1, lo1);
+        c0 = xor3(hi1, c1, k0);
+        c1 = lo1;
+        c2 = xor3(hi0, c3, k1);
+        c3 = lo0;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    v4u o = {c0, c1, c2, c3};
+    return o;
+}
+
+// Keep decisions of two scores at once: p2 holds their probabilities as packed fp16, w the two 16-bit Philox fields in the
+// same halves, sub2 = threshold - 1 in both halves (threshold >= 1).  A saturating subtraction leaves a half non-zero
+// iff field >= threshold; clipped to 1 it multiplies the fp16 bit pattern as an integer: the pattern, or zero.  Three
+// packed instructions for two scores instead of a comparison and a select for each.
+// (inline asm: from the same thing written with vector types the compiler recovers the comparison and emits a compare,
+// a select and a byte permute per score)
+__device__ __forceinline__ uint32_t keep_pair(uint32_t p2, uint32_t w, uint32_t sub2)
+{
+    uint32_t x;
+    asm("v_pk_sub_u16 %0, %1, %2 clamp\n\tv_pk_min_u16 %0, %0, %3\n\tv_pk_mul_lo_u16 %0, %4, %0"
+        : "=&v"(x)
+        : "v"(w), "s"(sub2), "v"(0x00010001u), "v"(p2));
+    return x;
 }
 
 // 16-bit field f (0..7) of a Philox output

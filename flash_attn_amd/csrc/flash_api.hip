@@ -118,6 +118,7 @@ void fill_args(const flash_params* p, int splits, fa::FwdArgs* a)
     a->alibi_left = (p->alibi_slopes && (a->causal || a->wr == 0)) ? 1 : 0;
     a->scale_log2 = p->softmax_scale * fa::kLog2e;
     a->drop_thr = flash_dropout_threshold(p->dropout_p);
+    a->drop_sub2 = a->drop_thr > 0 ? (a->drop_thr - 1) * 0x00010001u : 0u;
     a->drop_rscale = 1.0f / (1.0f - p->dropout_p);
     a->seed_lo = (uint32_t)p->seed;
     a->seed_hi = (uint32_t)(p->seed >> 32);
@@ -133,6 +134,9 @@ int tiled_variant(const flash_params* p)
 {
     // A non-positive scale does not commute with the row maximum: only the element-wise instance scales first.
     int variant = (p->d % 8 == 0 && p->softmax_scale > 0.0f && !p->scores_out) ? 1 : 0;  // (the score dump lives there too)
+    // A dropout probability below 2^-16 has threshold 0 (every element kept, survivors still scaled): the vector
+    // instances apply the decisions with threshold - 1 and leave that case to the element-wise one.
+    if (p->dropout_p > 0.0f && flash_dropout_threshold(p->dropout_p) == 0) variant = 0;
     if (p->alibi_slopes) variant |= 2;
     if (p->dropout_p > 0.0f) variant |= 4;
     return variant;

@@ -497,6 +497,9 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                 // drop iff field < threshold, row sum left undropped (src/flash_forward.h:221-237); the survivors' factor
                 // 1/(1-p) is common to the whole row and multiplies O once in the epilogue instead of every score here
                 const uint32_t i_u = (uint32_t)row_i[nb];
+                // first-round Philox product of the head-slice word: the same for the whole work-group, so a scalar multiply
+                const uint64_t bh_prod = (uint64_t)0xCD9E8D57u * (uint64_t)(uint32_t)bh;
+                const uint32_t bh_hi = (uint32_t)(bh_prod >> 32), bh_lo = (uint32_t)bh_prod;
                 uint8_t* kout = a.keep_out ? a.keep_out + ((size_t)bh * Nq + row_i[nb]) * Nk : nullptr;
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
@@ -504,11 +507,24 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                     for (int q = 0; q < 2; ++q) {
                         // the lane's eight keys among the 16 from jg on: field f belongs to key jg + 8*(f>>2) + 4*g + (f&3)
                         const int jg = kb0 + 32 * kb + 16 * q;
-                        const v4u w = philox4x32_10(dropout_call((uint32_t)(jg + 4 * g)), i_u, (uint32_t)bh, a.off_lo, a.seed_lo, a.seed_hi);
+                        const v4u w = philox4x32_10_c2(dropout_call((uint32_t)(jg + 4 * g)), i_u, bh_hi, bh_lo, a.off_lo, a.seed_lo, a.seed_hi);
+                        if constexpr (kVec) {
+                            // registers 8q + 2k and 8q + 2k + 1 become one packed fp16 word, fields 2k and 2k + 1 are the
+                            // halves of Philox word k: the decisions are applied to the packed word (keep_pair)
 #pragma unroll
-                        for (int f = 0; f < 8; ++f) {
-                            const int r = 8 * q + f;
-                            s[kb][nb][r] = philox_field16(w, f) >= a.drop_thr ? s[kb][nb][r] : 0.0f;
+                            for (int k = 0; k < 4; ++k) {
+                                union { v2h h; uint32_t u; } pk;
+                                pk.h = pack_f16(s[kb][nb][8 * q + 2 * k], s[kb][nb][8 * q + 2 * k + 1]);
+                                pk.u = keep_pair(pk.u, w[k], a.drop_sub2);
+                                pf[kb][q][nb][2 * k] = pk.h[0];
+                                pf[kb][q][nb][2 * k + 1] = pk.h[1];
+                            }
+                        } else {
+#pragma unroll
+                            for (int f = 0; f < 8; ++f) {
+                                const int r = 8 * q + f;
+                                s[kb][nb][r] = philox_field16(w, f) >= a.drop_thr ? s[kb][nb][r] : 0.0f;
+                            }
                         }
                         if (a.keep_out != nullptr) {  // debug dump: one uniform branch per call, none per score
 #pragma unroll
@@ -519,16 +535,18 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                         }
                     }
             }
+            if constexpr (!(kDropout && kVec)) {  // (there the dropout step has packed them already)
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+                for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int tt = 0; tt < 2; ++tt)
+                    for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-                    for (int e = 0; e < 8; e += 2) {
-                        const v2h h2 = pack_f16(s[kb][nb][8 * tt + e], s[kb][nb][8 * tt + e + 1]);
-                        pf[kb][tt][nb][e] = h2[0];
-                        pf[kb][tt][nb][e + 1] = h2[1];
-                    }
+                        for (int e = 0; e < 8; e += 2) {
+                            const v2h h2 = pack_f16(s[kb][nb][8 * tt + e], s[kb][nb][8 * tt + e + 1]);
+                            pf[kb][tt][nb][e] = h2[0];
+                            pf[kb][tt][nb][e + 1] = h2[1];
+                        }
+            }
         }
     };
 

@@ -406,6 +406,9 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         l_run += rs;
         if constexpr (kDropout) {
             const uint32_t i_u = (uint32_t)row_i;
+            // first-round Philox product of the head-slice word: the same for the whole work-group, so a scalar multiply
+            const uint64_t bh_prod = (uint64_t)0xCD9E8D57u * (uint64_t)(uint32_t)bh;
+            const uint32_t bh_hi = (uint32_t)(bh_prod >> 32), bh_lo = (uint32_t)bh_prod;
             uint8_t* kout = a.keep_out ? a.keep_out + ((size_t)bh * Nq + row_i) * Nk : nullptr;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
@@ -413,11 +416,15 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
                 for (int q = 0; q < 2; ++q) {
                     // the lane's eight keys among the 16 from jg on: field f belongs to key jg + 8*(f>>2) + 4*g + (f&3)
                     const int jg = kb0 + 32 * kb + 16 * q;
-                    const v4u w = philox4x32_10(dropout_call((uint32_t)(jg + 4 * g)), i_u, (uint32_t)bh, a.off_lo, a.seed_lo, a.seed_hi);
+                    const v4u w = philox4x32_10_c2(dropout_call((uint32_t)(jg + 4 * g)), i_u, bh_hi, bh_lo, a.off_lo, a.seed_lo, a.seed_hi);
+                    // the decisions are applied to the packed fp16 words (keep_pair); the 1/(1-p) waits for the epilogue
 #pragma unroll
-                    for (int f = 0; f < 8; ++f) {
-                        const int r = 8 * q + f;
-                        s[kb][r] = philox_field16(w, f) >= a.drop_thr ? s[kb][r] : 0.0f;  // the 1/(1-p) waits for the epilogue
+                    for (int k = 0; k < 4; ++k) {
+                        union { v2h h; uint32_t u; } pk;
+                        pk.h = pack_f16(s[kb][8 * q + 2 * k], s[kb][8 * q + 2 * k + 1]);
+                        pk.u = keep_pair(pk.u, w[k], a.drop_sub2);
+                        pf[kb][q][2 * k] = pk.h[0];
+                        pf[kb][q][2 * k + 1] = pk.h[1];
                     }
                     if (a.keep_out != nullptr) {  // debug dump: one uniform branch per call, none per score
 #pragma unroll
@@ -428,16 +435,18 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
                     }
                 }
         }
+        if constexpr (!kDropout) {  // (there the dropout step has packed them already)
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+            for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
+                for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-                for (int e = 0; e < 8; e += 2) {
-                    const v2h h2 = pack_f16(s[kb][8 * tt + e], s[kb][8 * tt + e + 1]);
-                    pf[kb][tt][e] = h2[0];
-                    pf[kb][tt][e + 1] = h2[1];
-                }
+                    for (int e = 0; e < 8; e += 2) {
+                        const v2h h2 = pack_f16(s[kb][8 * tt + e], s[kb][8 * tt + e + 1]);
+                        pf[kb][tt][e] = h2[0];
+                        pf[kb][tt][e + 1] = h2[1];
+                    }
+        }
     };
 
     // One iteration.  The four stage pointers are distinct LDS regions; declaring them restrict is what lets the
