@@ -91,13 +91,15 @@ constexpr float kLazyTau = 8.0f;
 // variant bits of the kernel template
 // kVarStamp: debug time stamps.  kVarAlibiLeft (with kVarAlibi, kVarVec): every visible key lies at or left of its row
 // (causal mask or a right window of 0), which lets the bias ride in the MFMA accumulator (see calib below).
-constexpr int kVarVec = 1, kVarAlibi = 2, kVarDropout = 4, kVarFullD = 8, kVarStamp = 16, kVarAlibiLeft = 32;
+// kVarKvOnce (with kVarVec, kVarFullD, no other feature): every K/V tile is requested by this work-group alone -- one row
+// block per slice and one query head per K/V head, the shape of a decode launch -- and its requests are non-temporal.
+constexpr int kVarVec = 1, kVarAlibi = 2, kVarDropout = 4, kVarFullD = 8, kVarStamp = 16, kVarAlibiLeft = 32, kVarKvOnce = 64;
 
 template <int D, int NB, int VAR>
 __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 0 ? 3 : 2) : 1) fwd_kernel(const FwdArgs a)
 {
     constexpr bool kVec = (VAR & kVarVec) != 0, kAlibi = (VAR & kVarAlibi) != 0, kDropout = (VAR & kVarDropout) != 0,
-                   kFullD = (VAR & kVarFullD) != 0, kStamp = (VAR & kVarStamp) != 0;
+                   kFullD = (VAR & kVarFullD) != 0, kStamp = (VAR & kVarStamp) != 0, kKvOnce = (VAR & kVarKvOnce) != 0;
     using C = FwdCfg<D, NB>;
     Stamps<kStamp> stamps;
     stamps.take(0);
@@ -269,18 +271,21 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
         FA_LDS char* const vst = (FA_LDS char*)smem + NSTG * C::KBUF + stage * C::VBUF;
         const char* const Kb = reinterpret_cast<const char*>(Kbh);
         const char* const Vb = reinterpret_cast<const char*>(Vbh);
+        // (kKvOnce: a stream that only this work-group reads is requested non-temporal)
 #pragma unroll
         for (int i = 0; i < C::NKX; ++i) {
             if (i == C::NKX - 1 && !k_extra) break;
             uint32_t o = koff[i] + tb;
             if (rows_left < BC && krow[i] >= rows_left) o -= (uint32_t)((krow[i] - rows_left + 1) * D * 2);
-            dma_kib(Kb, o, kst + (wave + 4 * i) * 1024);
+            if constexpr (kKvOnce) dma_kib_nt(Kb, o, kst + (wave + 4 * i) * 1024);
+            else dma_kib(Kb, o, kst + (wave + 4 * i) * 1024);
         }
 #pragma unroll
         for (int i = 0; i < C::NVX; ++i) {
             uint32_t o = voff[i] + tb;
             if (rows_left < BC && vrow[i] >= rows_left) o -= (uint32_t)((vrow[i] - rows_left + 1) * D * 2);
-            dma_kib(Vb, o, vst + (wave + 4 * i) * 1024);
+            if constexpr (kKvOnce) dma_kib_nt(Vb, o, vst + (wave + 4 * i) * 1024);
+            else dma_kib(Vb, o, vst + (wave + 4 * i) * 1024);
         }
     };
     // wait until at most the requests of one tile (the youngest) are still in flight / until none is
@@ -805,7 +810,8 @@ inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
         e = launch_fwd_instance<D, NB, ST | kVarAlibi | kVarDropout>(a, st);
     } else if (a.d == D) {
         constexpr int V = ST | kVarVec | kVarFullD;
-        if (feat == 0) e = launch_fwd_instance<D, NB, V>(a, st);
+        const bool kv_once = ST == 0 && a.Tr == 1 && a.kv_group == 1;
+        if (feat == 0) e = kv_once ? launch_fwd_instance<D, NB, V | (ST == 0 ? kVarKvOnce : 0)>(a, st) : launch_fwd_instance<D, NB, V>(a, st);
         else if (feat == kVarAlibi) e = a.alibi_left ? launch_fwd_instance<D, NB, V | AL>(a, st) : launch_fwd_instance<D, NB, V | kVarAlibi>(a, st);
         else if (feat == kVarDropout) e = launch_fwd_instance<D, NB, V | kVarDropout>(a, st);
         else e = a.alibi_left ? launch_fwd_instance<D, NB, V | AL | kVarDropout>(a, st) : launch_fwd_instance<D, NB, V | kVarAlibi | kVarDropout>(a, st);
