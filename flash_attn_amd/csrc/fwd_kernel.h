@@ -265,28 +265,39 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     }
     const bool k_extra = wave + 4 * (C::NKX - 1) <= CH;  // the last round of K blocks exists for this wave
     auto dma_tile = [&](int tile, int stage) {
-        const uint32_t tb = (uint32_t)tile * (uint32_t)(BC * D * 2);
-        const int rows_left = Nk - tile * BC;  // >= 1; keys past Nk re-read key Nk - 1 (their scores are masked)
+        // The tile's offset joins the scalar base address, so that a request of a whole tile needs no vector
+        // arithmetic at all; only the last tile of a ragged sequence adjusts rows: keys past Nk re-read key Nk - 1
+        // (their scores are masked).
+        const size_t tb = (size_t)tile * (size_t)(BC * D * 2);
+        const int rows_left = Nk - tile * BC;  // >= 1
         FA_LDS char* const kst = (FA_LDS char*)smem + stage * C::KBUF;
         FA_LDS char* const vst = (FA_LDS char*)smem + NSTG * C::KBUF + stage * C::VBUF;
-        const char* const Kb = reinterpret_cast<const char*>(Kbh);
-        const char* const Vb = reinterpret_cast<const char*>(Vbh);
-        // (kKvOnce: a stream that only this work-group reads is requested non-temporal)
+        const char* const Kb = reinterpret_cast<const char*>(Kbh) + tb;
+        const char* const Vb = reinterpret_cast<const char*>(Vbh) + tb;
+        auto issue = [&](auto ragged_c) {
+            constexpr bool kRagged = decltype(ragged_c)::value;
+            // (laundered: the compiler otherwise carries one running vector offset per request through every tile
+            // for the sake of this one)
+            int rows_left = Nk - tile * BC;
+            if constexpr (kRagged) asm volatile("" : "+s"(rows_left));
 #pragma unroll
-        for (int i = 0; i < C::NKX; ++i) {
-            if (i == C::NKX - 1 && !k_extra) break;
-            uint32_t o = koff[i] + tb;
-            if (rows_left < BC && krow[i] >= rows_left) o -= (uint32_t)((krow[i] - rows_left + 1) * D * 2);
-            if constexpr (kKvOnce) dma_kib_nt(Kb, o, kst + (wave + 4 * i) * 1024);
-            else dma_kib(Kb, o, kst + (wave + 4 * i) * 1024);
-        }
+            for (int i = 0; i < C::NKX; ++i) {
+                if (i == C::NKX - 1 && !k_extra) break;
+                uint32_t o = koff[i];
+                if (kRagged && krow[i] >= rows_left) o -= (uint32_t)((krow[i] - rows_left + 1) * D * 2);
+                if constexpr (kKvOnce) dma_kib_nt(Kb, o, kst + (wave + 4 * i) * 1024);
+                else dma_kib(Kb, o, kst + (wave + 4 * i) * 1024);
+            }
 #pragma unroll
-        for (int i = 0; i < C::NVX; ++i) {
-            uint32_t o = voff[i] + tb;
-            if (rows_left < BC && vrow[i] >= rows_left) o -= (uint32_t)((vrow[i] - rows_left + 1) * D * 2);
-            if constexpr (kKvOnce) dma_kib_nt(Vb, o, vst + (wave + 4 * i) * 1024);
-            else dma_kib(Vb, o, vst + (wave + 4 * i) * 1024);
-        }
+            for (int i = 0; i < C::NVX; ++i) {
+                uint32_t o = voff[i];
+                if (kRagged && vrow[i] >= rows_left) o -= (uint32_t)((vrow[i] - rows_left + 1) * D * 2);
+                if constexpr (kKvOnce) dma_kib_nt(Vb, o, vst + (wave + 4 * i) * 1024);
+                else dma_kib(Vb, o, vst + (wave + 4 * i) * 1024);
+            }
+        };
+        if (rows_left >= BC) issue(std::false_type{});
+        else issue(std::true_type{});
     };
     // wait until at most the requests of one tile (the youngest) are still in flight / until none is
     auto dma_wait = [&](bool one_tile_in_flight) {

@@ -187,16 +187,25 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     }
     const char* const Kb = reinterpret_cast<const char*>(Kbh);
     const char* const Vb = reinterpret_cast<const char*>(Vbh);
-    // tile index t counts from tile_begin; keys past Nk re-read key Nk - 1 (their scores are masked)
+    // tile index t counts from tile_begin; keys past Nk re-read key Nk - 1 (their scores are masked).  The tile's
+    // offset joins the scalar base address: a whole tile is requested without any vector arithmetic, only the last
+    // tile of a ragged sequence adjusts rows.
     auto load_tile = [&](const char* base, uint32_t go, int t, FA_LDS char* stage) {
-        const int rows_left = Nk - (tile_begin + t) * BC;  // >= 1
+        const char* const tbase = base + (size_t)t * (size_t)(BC * d * 2);
+        auto issue = [&](auto ragged_c) {
+            constexpr bool kRagged = decltype(ragged_c)::value;
+            int rows_left = Nk - (tile_begin + t) * BC;  // >= 1
+            if constexpr (kRagged) asm volatile("" : "+s"(rows_left));  // (no running vector offsets for this case)
 #pragma unroll
-        for (int x = 0; x < NKL; ++x) {
-            const int key = dkey + 32 * x;
-            uint32_t o = go + (uint32_t)t * (uint32_t)(BC * d * 2) + (uint32_t)(32 * x * d * 2);
-            if (rows_left < BC && key >= rows_left) o -= (uint32_t)((key - rows_left + 1) * d * 2);
-            dma_kib(base, o, stage + (wave + 8 * x) * 1024);
-        }
+            for (int x = 0; x < NKL; ++x) {
+                const int key = dkey + 32 * x;
+                uint32_t o = go + (uint32_t)(32 * x * d * 2);
+                if (kRagged && key >= rows_left) o -= (uint32_t)((key - rows_left + 1) * d * 2);
+                dma_kib(tbase, o, stage + (wave + 8 * x) * 1024);
+            }
+        };
+        if (Nk - (tile_begin + t) * BC >= BC) issue(std::false_type{});
+        else issue(std::true_type{});
     };
     static_assert(NKL == NVL, "K and V tiles have the same shape");
     auto load_k = [&](int t, FA_LDS char* stage) { load_tile(Kb, kgo, t, stage); };
