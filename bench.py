@@ -199,6 +199,13 @@ def stage_timeline(fa, c, q, k, v):
            "tiles_per_group": {"mean": float(tiles.mean()), "max": int(tiles.max())},
            "us_per_tile_in_loop": float(loop.sum() / max(1, int((tiles - 1).clip(min=0).sum()))),
            "epilogue_us": float((rel[:, 5] - rel[:, 4]).mean())}
+    # word 8: shader-clock cycles between the first barrier and the end of the loop -> the clock the CUs ran at there
+    span = (t[:, 5] - t[:, 3]) / 100.0
+    ok = span >= 3.0
+    if ok.any():
+        mhz = t[ok, 8] / span[ok]
+        out["loop_clock_mhz"] = {"mean": float(mhz.mean()), "min": float(mhz.min()), "max": float(mhz.max())}
+        out["shader_cycles_per_tile_in_loop"] = float(t[ok, 8].sum() / max(1, int(tiles[ok].sum())))
     xcc = (t[:, 7] >> 16) & 0xf
     cu_se = (t[:, 7] & 0xffff) >> 8  # CU, SH and SE fields of HW_ID
     out["distinct_cus"] = int(len(set(zip(xcc.tolist(), cu_se.tolist()))))
@@ -295,6 +302,9 @@ def main():
                     help="launches of the steady-state leg (the reference times 1000, src/main.cu:187-213); 0 = skip")
     ap.add_argument("--stage-timeline", action="store_true",
                     help="print the per-stage timeline of the headline workload (instrumented kernel instance) and exit")
+    ap.add_argument("--zero-inputs", action="store_true",
+                    help="diagnostic: all-zero Q, K, V instead of N(0,1) (same instruction stream; the power management "
+                         "then leaves the clock high -- compare loop_clock_mhz of --stage-timeline); never a valid rate")
     ap.add_argument("--grid", action="store_true",
                     help="print a table of forward rates over sequence lengths 512 ... 16384 at 16384 tokens per launch "
                          "(d = 128 with 16 heads, d = 64 with 32; plain and causal) and exit")
@@ -328,6 +338,9 @@ def main():
     name = args.workload
     c = CONFIGS[name] if name in CONFIGS else DIAG[name]
     q, k, v = make_inputs(c)
+    if args.zero_inputs:
+        for t in (q, k, v):
+            t.zero_()
     if args.stage_timeline:
         print(json.dumps({"workload": f"{name}: {DESCR[name]}", "stage_timeline": stage_timeline(fa, c, q, k, v)}))
         return
@@ -370,7 +383,8 @@ def main():
     result = {
         "metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": host_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
-        "data": "synthetic", "config": {"workload": f"{name}: {DESCR[name]}", "inputs": "fp16 RN(N(0,1)), seeded, resident in HBM",
+        "data": "synthetic", "config": {"workload": f"{name}: {DESCR[name]}", "inputs": ("ALL ZERO (diagnostic run, not a valid rate)" if args.zero_inputs
+                                                   else "fp16 RN(N(0,1)), seeded, resident in HBM"),
                                         "accumulate": "fp32", "outputs": "fp16 O + fp32 LSE"},
         "roofline": roof,
     }

@@ -14,7 +14,7 @@ _LIB_PATH = os.path.join(_HERE, "lib", "libflash_attn_mi355.so")
 FLASH_OK = 0
 FLASH_MAX_HEAD_DIM = 128
 FLASH_MAX_SPLITS = 128
-FLASH_STAMP_WORDS = 8
+FLASH_STAMP_WORDS = 9
 FLASH_STATIC_SCRATCH_BYTES = 32 << 20
 KERNEL_AUTO, KERNEL_4WAVE, KERNEL_8WAVE = 0, 1, 2
 
@@ -171,7 +171,7 @@ def flash_forward(q, k, v, softmax_scale=None, causal=False, window=(-1, -1), al
     return_keep_mask, the uint8 keep decisions [B,H,Nq,Nk] the kernel applied.  scores_out: optional fp32
     [B,H,Nq,Nk] tensor (pre-filled with -inf) that receives the visible scores (debug; slow kernel instance).
     kernel_hint: KERNEL_AUTO / KERNEL_4WAVE / KERNEL_8WAVE.  return_stage_stamps: also return the per-work-group
-    time stamps [groups, 8] int64 of the instrumented kernel instance (debug), as the last element."""
+    time stamps [groups, FLASH_STAMP_WORDS] int64 of the instrumented kernel instance (debug), as the last element."""
     import torch
 
     B, H, Nq, Nk, d = _check_qkv(q, k, v)
@@ -261,9 +261,9 @@ def num_splits_heuristic(batch_nheads_mblocks, num_cus, num_n_blocks, max_splits
 
 
 def stage_stamp_names():
-    """Meaning of the eight words of a stage-stamp row (see stage_stamps_out in the header)."""
+    """Meaning of the nine words of a stage-stamp row (see stage_stamps_out in the header)."""
     return ("entry", "requests_issued", "requests_landed", "first_barrier", "first_scores", "loop_done", "stored",
-            "tiles<<32|xcc<<16|hw_id")
+            "tiles<<32|xcc<<16|hw_id", "shader_cycles_first_barrier_to_loop_done")
 
 
 def _shape_params(B, H, Nq, Nk, d, num_splits):

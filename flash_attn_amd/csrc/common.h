@@ -72,10 +72,14 @@ __device__ __forceinline__ float xhalf_sum(float v)
 
 // Debug time stamps of the instrumented kernel instances: readings of the constant 100 MHz counter, taken by every wave
 // (they are scalar) and stored by the first lane of the work-group in the epilogue with an ordinary vector store.
-constexpr int kStampWords = 8;  // FLASH_STAMP_WORDS of the public header
+// Beside stages 3 and 5 the shader-clock counter is read as well: their difference over the time between the two stages
+// is the clock the work-group ran at in its key-tile loop.
+constexpr int kStampTimes = 7;
+constexpr int kStampWords = 9;  // FLASH_STAMP_WORDS of the public header
 template <bool kOn>
 struct Stamps {
-    uint64_t t[kOn ? kStampWords - 1 : 1];
+    uint64_t t[kOn ? kStampTimes : 1];
+    uint64_t cyc[kOn ? 2 : 1];
     // stage 0 also presets the later stages: one that a work-group never reaches (no key tile) is stored as the time
     // of the stage before it
     __device__ __forceinline__ void take(int i)
@@ -84,13 +88,17 @@ struct Stamps {
             const uint64_t now = __builtin_amdgcn_s_memrealtime();
             if (i == 0) {
 #pragma unroll
-                for (int k = 0; k < kStampWords - 1; ++k) t[k] = now;
+                for (int k = 0; k < kStampTimes; ++k) t[k] = now;
+                cyc[0] = cyc[1] = 0;
             } else {
                 t[i] = now;
+                if (i == 3) cyc[0] = __builtin_amdgcn_s_memtime();
+                if (i == 5) cyc[1] = __builtin_amdgcn_s_memtime();
             }
         }
     }
-    // word 7: tiles << 32 | XCC id << 16 | low half of HW_ID (wave, SIMD, pipe, CU, SH, SE)
+    // word 7: tiles << 32 | XCC id << 16 | low half of HW_ID (wave, SIMD, pipe, CU, SH, SE); word 8: shader-clock cycles
+    // between stages 3 and 5
     __device__ __forceinline__ void store(uint64_t* out, int ntiles) const
     {
         if constexpr (kOn) {
@@ -100,11 +108,12 @@ struct Stamps {
                 uint64_t* o = out + (size_t)blockIdx.x * kStampWords;
                 uint64_t last = t[0];
 #pragma unroll
-                for (int i = 0; i < kStampWords - 1; ++i) {
+                for (int i = 0; i < kStampTimes; ++i) {
                     last = t[i] > last ? t[i] : last;
                     o[i] = last;
                 }
-                o[kStampWords - 1] = ((uint64_t)(uint32_t)ntiles << 32) | ((uint64_t)(xcc & 0xfu) << 16) | (hw & 0xffffu);
+                o[kStampTimes] = ((uint64_t)(uint32_t)ntiles << 32) | ((uint64_t)(xcc & 0xfu) << 16) | (hw & 0xffffu);
+                o[kStampTimes + 1] = cyc[1] > cyc[0] ? cyc[1] - cyc[0] : 0;
             }
         }
     }

@@ -96,14 +96,16 @@ typedef struct flash_params {
      * at stage_stamps_out + FLASH_STAMP_WORDS * blockIdx (buffer size: flash_stage_stamps_bytes): words 0..6 are readings
      * of the constant 100 MHz device counter -- 0 entry, 1 all prologue requests issued, 2 own requests landed,
      * 3 first work-group barrier passed, 4 first score tile computed, 5 key-tile loop finished, 6 results stored --
-     * and word 7 packs (tiles of the work-group) << 32 | hardware id of the CU (bits 0-15 of HW_ID; bits 16-19 the
-     * XCC).  The call then runs instrumented instances of the same kernels (same arithmetic, same results).  With a
+     * word 7 packs (tiles of the work-group) << 32 | hardware id of the CU (bits 0-15 of HW_ID; bits 16-19 the
+     * XCC), and word 8 is the number of shader-clock cycles (s_memtime) between readings 3 and 5: divided by their
+     * distance in time it is the clock the CU ran at while the work-group was in its key-tile loop (the power
+     * management lowers it when the MFMA operands change from instruction to instruction).  The call then runs instrumented instances of the same kernels (same arithmetic, same results).  With a
      * split count above 1 the combine step is not stamped.  The only instrumentation of the reference is the event
      * pair around its launches (src/main.cu:195-213). */
     uint64_t *stage_stamps_out;
 } flash_params;
 
-#define FLASH_STAMP_WORDS 8
+#define FLASH_STAMP_WORDS 9
 
 /* Tiled forward over the whole key range: replaces
  *     forward_kernel<...><<<dim3(Tr,H,B),256,smem>>>(param)              (src/flash_forward.h:13-15, src/main.cu:189)

@@ -307,6 +307,13 @@ def test_stage_stamps(fa, oracle, hint, N, d, kw):
     assert ((t[:, 6] - t[:, 0]) < 100_000_000).all()  # less than a second
     tiles = t[:, 7] >> 32
     assert tiles.min() >= 1 and tiles.max() <= (N + 63) // 64
+    # word 8: shader-clock cycles between stamps 3 and 5; over their distance in time a plausible clock (the 100 MHz
+    # counter resolves 10 ns, so only work-groups that spent a few microseconds there are judged)
+    dt = (t[:, 5] - t[:, 3]) / 100.0
+    long_enough = dt >= 3.0
+    if long_enough.any():
+        mhz = t[long_enough, 8] / dt[long_enough]
+        assert mhz.min() > 300 and mhz.max() < 3500, mhz
     # split entry point: one stamp row per work-group of the split launch
     o, l, st2 = fa.flash_forward_splitkv(q, k, v, num_splits=2, kernel_hint=hint, return_stage_stamps=True, **kw)
     check_o_lse(o, l, O, L, "instrumented split instance")
