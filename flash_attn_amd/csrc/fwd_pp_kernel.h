@@ -463,8 +463,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     auto iteration = [&](auto last_c, FA_LDS const char* __restrict__ rdv, FA_LDS const char* __restrict__ rdk,
                          FA_LDS char* __restrict__ wrk, FA_LDS char* __restrict__ wrv, int t) __attribute__((always_inline)) {
         const int kb0 = (tile_begin + t) * BC;
-        // ---------------- VALU phase: request the tiles to come, softmax of tile t
-        if (t + 3 < ntiles) load_k(t + 3, wrk);
+        // ---------------- VALU phase: request the V tile to come, softmax of tile t
         if (t + 2 < ntiles) load_v(t + 2, wrv);
         const int mask_sides = (kb0 < lo_max ? 1 : 0) | (kb0 + BC - 1 > hi_min ? 2 : 0);
         softmax(mask_sides, kb0);
@@ -479,7 +478,15 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         __builtin_amdgcn_s_setprio(1);
         mfma_phase(last_c, vbase, kbase);
         __builtin_amdgcn_s_setprio(0);
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of K(t+3), V(t+2) is in LDS
+        // K(t+3) is requested here, behind the wave's last MFMA of the phase (the four waves of a group reach the start
+        // of their VALU phase together: requests issued there queue up in front of the softmax), and waited for one
+        // iteration later: what must have landed now is K(t+2), requested an iteration ago, and V(t+2).
+        if (t + 3 < ntiles) {
+            load_k(t + 3, wrk);
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NKL) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
         lds_barrier();
     };
 
@@ -539,10 +546,14 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     // Tiles whose keys (and whose successor's keys) are all invisible to this wave contribute nothing: there the wave
     // only serves its share of the loads and the barriers.  Live tiles form one contiguous range [t_lo, t_hi).
     auto idle_iteration = [&](int t) {
-        if (t + 3 < ntiles) load_k(t + 3, Ks + ((t + 3) % NST) * C::KBUF);
         if (t + 2 < ntiles) load_v(t + 2, Vs + ((t + 2) % NST) * C::VBUF);
         lds_barrier();
-        __builtin_amdgcn_s_waitcnt(0x0F70);
+        if (t + 3 < ntiles) {
+            load_k(t + 3, Ks + ((t + 3) % NST) * C::KBUF);
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NKL) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
         lds_barrier();
     };
     // The full loop starts one tile before the first visible one: that tile is masked entirely (whatever stale scores
