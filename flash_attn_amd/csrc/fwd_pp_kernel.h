@@ -15,9 +15,10 @@
 //    a request covers four whole rows of global memory and the fragment reads (ds_read_b128 for K, ds_read_b64_tr_b16
 //    for V) are free of bank conflicts; a fragment address is one base register ^ constant plus an immediate.
 //    Q and O go through 8 KiB of wave-private LDS in the same layout, for the same reason (whole rows per request).
-//  * Four LDS stages per tensor: K(t+3) and V(t+2) are requested at the start of the VALU phase of iteration t and
-//    waited for (vmcnt) at the end of the MFMA phase of the same iteration; with the half-iteration offset their
-//    slots (K(t-1), V(t-2)) were last read two barriers earlier, and the first reader comes two barriers later.
+//  * Four LDS stages per tensor: V(t+2) is requested at the start of the VALU phase of iteration t and waited for (vmcnt)
+//    at the end of its MFMA phase; K(t+3) is requested at the end of that MFMA phase and waited for at the end of the next
+//    one.  With the half-iteration offset of the wave groups their slots (K(t-1), V(t-2)) were last read at least two
+//    barriers before the request, and the first reader comes at least one barrier after the wait of the later group.
 //  * Barriers wait for LDS traffic only; the first V fragment reads of a phase are issued before its barrier.
 #pragma once
 #include "fwd_kernel.h"
