@@ -141,6 +141,29 @@ def test_dropout_mask_bit_exact_and_output(fa, oracle, shape):
         assert torch.equal(o, o2)
 
 
+@pytest.mark.parametrize("shape", [(1, 2, 300, 300, 128), (1, 2, 150, 150, 64)])
+def test_dropout_threshold_edges(fa, oracle, shape):
+    """The smallest thresholds: p below 2^-16 has threshold 0 (every element kept, survivors still scaled by 1/(1-p)) and
+    is served by the element-wise instance; p = 2^-16 has threshold 1, the smallest one the vector instances' packed
+    keep decisions (saturating subtraction of threshold - 1) see; p close to 1 the largest."""
+    import torch
+    B, H, Nq, Nk, d = shape
+    q, k, v = _qkv(B, H, Nq, Nk, d, seed=sum(shape) + 1)
+    for p in (1e-6, 2.0 ** -16, 3.0 * 2.0 ** -16, 1.0 - 2.0 ** -15):
+        o, lse, km = fa.flash_forward(q, k, v, causal=True, dropout_p=p, seed=5, offset=9, return_keep_mask=True)
+        keep = oracle.dropout_keep_mask(5, 9, p, B, H, Nq, Nk)
+        vis = np.tril(np.ones((Nq, Nk), dtype=bool))  # the dump covers the pairs the mask leaves visible
+        assert np.array_equal(km.cpu().numpy()[..., vis], keep[..., vis]), f"p={p}"
+        if p == 1e-6:
+            assert keep.all()
+        O, L = oracle_forward_batched(oracle, q, k, v, causal=True, keep_mask=torch.from_numpy(keep), p_drop=p)
+        if p < 0.5:
+            check_o_lse(o, lse, O, L, f"dropout p={p} {shape}")
+        else:  # survivors are scaled by 32768: compare relative to that
+            assert np.allclose(lse.cpu().numpy(), L, atol=1e-4)
+            assert np.allclose(o.float().cpu().numpy() * (1 - p), O * (1 - p), atol=2e-3, rtol=1e-2)
+
+
 @pytest.mark.parametrize("S", [1, 2, 3, 5, 8])
 def test_general_splitkv_matches_unsplit(fa, oracle, S):
     """The reference's split path for Nq > 1 (its checked-in run: N=1021, d=31, src/main.cu:39-49) with every mask;
