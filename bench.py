@@ -370,7 +370,20 @@ def main():
         roof["steady_state"] = {"launches": args.steady_launches, "ms": st_ms, "achieved": ach, "unit": roof["unit"],
                                 "frac": ach / roof["peak"]}
     if roof["bound"] == "mfma" and not args.only_main:
-        # `peak` is the published figure; what the MFMA pipe of this GPU sustains on changing random operands (with no
+        # `peak` is the published figure: 256 CUs x 4 SIMDs x 1024 flop per cycle x 2.4 GHz.  The clock the kernel is
+        # allowed on this data is read from inside it (stage stamps of one instrumented launch, taken while the GPU
+        # is still warm from the timed legs): shader cycles of the work-groups' loops over the time they took.
+        roof["peak_basis"] = {"cus": 256, "simds_per_cu": 4, "flop_per_simd_cycle": 1024, "clock_ghz": 2.4}
+        try:
+            tl = stage_timeline(fa, c, q, k, v)
+            if "loop_clock_mhz" in tl:
+                clk = tl["loop_clock_mhz"]["mean"]
+                roof["loop_clock_mhz"] = clk
+                roof["frac_of_peak_at_loop_clock"] = roof["achieved"] / (PEAK_F16_TFLOPS * clk / 2400.0)
+        except Exception as e:  # a diagnostic: the line is valid without it
+            roof["loop_clock_mhz"] = None
+            print(f"bench.py: stage stamps unavailable ({e})", file=sys.stderr)
+        # what the MFMA pipe of this GPU sustains on changing random operands (with no
         # other work at all) is measured beside it, since the power management makes it data dependent
         sus = mfma_sustained()
         if sus:
