@@ -96,6 +96,24 @@ def test_live_reference_bit_exact(oracle):
         assert oracle.num_splits_heuristic(*args) == oracle.ref_num_splits_heuristic(*args)
 
 
+def test_live_reference_expresses_left_window_as_causal_plus_symmetric(oracle):
+    """The reference's CPU function has no (left, right) window, but its causal mask on top of its symmetric window
+    leaves exactly the keys i - left <= j <= i (src/main.cu:330-349): the benchmark times it that way as the CPU
+    baseline of the sliding-window + ALiBi configuration.  Bit-exact against the restatement's window (left, 0)."""
+    if oracle.ref_lib() is None:
+        pytest.skip("oracle/_ref not built (reference checkout absent)")
+    rng = np.random.default_rng(8)
+    B, H, N, d = 1, 3, 150, 64
+    q, k, v = rand_qkv(rng, B, H, N, N, d)
+    sl = oracle.alibi_slopes(H)
+    scale = np.float32(1.0 / np.sqrt(d))
+    for left in (0, 5, 64, 149, 400):
+        for s in (None, sl):
+            R = oracle.ref_attention_forward_cpu(q, k, v, scale, causal=True, window_size=left, slopes=s)
+            O, _ = oracle.attention_forward(q, k, v, scale, window=(left, 0), slopes=s, nthreads=2, skip_masked=False)
+            assert np.array_equal(O, R), (left, s is not None)
+
+
 # ------------------------------------------------------------------------------------------ brute force / closed forms
 @pytest.mark.parametrize("shape", [(1, 2, 8, 8, 4), (2, 2, 17, 17, 24), (1, 3, 5, 29, 16), (1, 1, 40, 13, 8), (1, 2, 1, 300, 32)])
 def test_brute_force_all_features(oracle, shape):
