@@ -20,5 +20,7 @@ from .binding import (  # noqa: F401
     KERNEL_4WAVE,
     KERNEL_8WAVE,
     FLASH_STAMP_WORDS,
+    FLASH_STATIC_SCRATCH_BYTES,
+    FLASH_MAX_SPLITS,
     lib,
 )

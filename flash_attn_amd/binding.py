@@ -91,6 +91,8 @@ def lib():
         L.flash_last_hip_error.restype = C.c_char_p
         L.flash_strerror.restype = C.c_char_p
         L.flash_strerror.argtypes = [C.c_int]
+        L.flash_params_init.restype = None
+        L.flash_params_init.argtypes = [pp]
         L.flash_params_size.restype = C.c_size_t
         if L.flash_params_size() != C.sizeof(FlashParams):
             raise ImportError(f"{_LIB_PATH} was built with another flash_params ({L.flash_params_size()} bytes, this "
@@ -130,6 +132,7 @@ def make_params(q, k, v, o, lse, softmax_scale=None, causal=False, window=(-1, -
                 scores_out=None, kernel_hint=KERNEL_AUTO):
     B, H, Nq, Nk, d = _check_qkv(q, k, v)
     p = FlashParams()
+    lib().flash_params_init(C.byref(p))
     p.Q, p.K, p.V, p.O, p.LSE = _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse)
     p.O_partial, p.LSE_partial = _ptr(o_partial), _ptr(lse_partial)
     p.B, p.H, p.Nq, p.Nk, p.d = B, H, Nq, Nk, d
@@ -266,25 +269,30 @@ def stage_stamp_names():
             "tiles<<32|xcc<<16|hw_id", "shader_cycles_first_barrier_to_loop_done")
 
 
-def _shape_params(B, H, Nq, Nk, d, num_splits):
+def _shape_params(B, H, Nq, Nk, d, num_splits, causal=False, window=(-1, -1), H_kv=0):
     p = FlashParams()
+    lib().flash_params_init(C.byref(p))
     p.B, p.H, p.Nq, p.Nk, p.d = B, H, Nq, Nk, d
     p.softmax_scale = 1.0
     p.num_splits = num_splits
-    p.window_left = p.window_right = -1
+    p.is_causal = int(bool(causal))
+    p.window_left, p.window_right = int(window[0]), int(window[1])
+    p.H_kv = int(H_kv)
     return p
 
 
-def resolve_splits(B, H, Nq, Nk, d, num_splits=0):
-    rc = lib().flash_splitkv_resolve_splits(C.byref(_shape_params(B, H, Nq, Nk, d, num_splits)))
+def resolve_splits(B, H, Nq, Nk, d, num_splits=0, causal=False, window=(-1, -1), H_kv=0):
+    """The split count flash_forward_splitkv will use for such a call (num_splits <= 0: the library's choice)."""
+    rc = lib().flash_splitkv_resolve_splits(C.byref(_shape_params(B, H, Nq, Nk, d, num_splits, causal, window, H_kv)))
     if rc < 0:
         raise FlashError(rc, "flash_splitkv_resolve_splits")
     return rc
 
 
-def workspace_bytes(B, H, Nq, Nk, d, num_splits=0):
+def workspace_bytes(B, H, Nq, Nk, d, num_splits=0, causal=False, window=(-1, -1), H_kv=0):
     ob, lb = C.c_size_t(), C.c_size_t()
-    rc = lib().flash_splitkv_workspace_bytes(C.byref(_shape_params(B, H, Nq, Nk, d, num_splits)), C.byref(ob), C.byref(lb))
+    rc = lib().flash_splitkv_workspace_bytes(C.byref(_shape_params(B, H, Nq, Nk, d, num_splits, causal, window, H_kv)),
+                                             C.byref(ob), C.byref(lb))
     if rc != FLASH_OK:
         raise FlashError(rc, "flash_splitkv_workspace_bytes")
     return ob.value, lb.value

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace fa {
 
 typedef _Float16 half_t;
@@ -49,13 +51,40 @@ struct FwdArgs {
     int Tr;              // number of query row blocks
     int kernel_hint;     // 0: by shape, 1: 4-wave kernel, 2: 8-wave kernel where it can serve the call
     int alibi_left;      // ALiBi and no visible key lies right of its row (causal, or right window 0)
-    int slice_chunk;     // 4-wave kernel: head slices per chunk of the work-group order (set by its launcher)
+    int slice_chunk;     // head slices per chunk of the work-group order (set by the kernel's launcher)
+    int snake_end;       // work-groups below this index sit on the GPU together; odd 256-blocks of them run reversed (launcher)
 
     // index of the K/V slice [Nk,d] read by query slice bh = b * H + h
     __device__ __forceinline__ int kv_slice(int bh) const { return (bh / H) * Hk + (bh % H) / kv_group; }
 };
 
 __device__ __forceinline__ int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// Position of a work-group in the launch's work order.  The order is "heaviest first", which balances a launch that
+// makes several rounds: whichever place frees up takes the heaviest work-group left.  But the work-groups of the first
+// round are not placed by load: the dispatcher deals work-group i to XCD i % 8 and there to CU (i / 8) % 32, so that with
+// r places per CU work-groups i, i + 256, ..., i + 256 (r - 1) share a CU whatever they weigh (measured: a causal launch
+// of 512 work-groups at two per CU left the CUs with 2 ... 32 key tiles each).  Inside that resident part (indices below
+// snake_end = min(work-groups, places), a multiple of 8) every second block of 256 therefore takes its items in reverse
+// CU order -- the CU with the heaviest item of one block gets the lightest of the next -- while i % 8, the XCD and with it
+// the L2 that a head slice's K and V sit in, stays as it is.
+__device__ __forceinline__ int work_position(int block, int snake_end)
+{
+    if (block < snake_end && (block & 256)) {
+        const int base = block & ~255;
+        const int size = snake_end - base < 256 ? snake_end - base : 256;  // a multiple of 8
+        const int pos = block - base;
+        return base + ((size >> 3) - 1 - (pos >> 3)) * 8 + (pos & 7);
+    }
+    return block;
+}
+
+// snake_end for a launch of `groups` work-groups with `resident` places on the GPU
+inline int snake_end_for(long long groups, int resident)
+{
+    const long long n = groups < resident ? groups : resident;
+    return (int)(n & ~7LL);
+}
 
 // Exchange between lane l and lane l^32 (v_permlane32_swap): result[0] holds the low half's value in both halves,
 // result[1] the high half's.
@@ -313,17 +342,19 @@ inline hipError_t launch_kernel(void (*kern)(P...), dim3 grid, dim3 block, size_
 }
 
 // Raises the dynamic-LDS limit of a kernel once per device (the attribute belongs to the device's copy of the kernel).
-// `done` is the caller's per-kernel flag array; concurrent first calls may both set the attribute, which is harmless.
+// `done` is the caller's per-kernel flag array.  Concurrent first calls from several threads may both set the
+// attribute, which is harmless; the flags are atomics so that such calls do not race in the language's sense either.
 constexpr int kMaxDevices = 64;
-inline hipError_t ensure_dynamic_lds(const void* kern, int bytes, bool (&done)[kMaxDevices])
+typedef std::atomic<bool> DeviceFlags[kMaxDevices];
+inline hipError_t ensure_dynamic_lds(const void* kern, int bytes, DeviceFlags& done)
 {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= kMaxDevices) dev = kMaxDevices - 1;  // beyond the table: set it on every launch
-    if (done[dev] && dev != kMaxDevices - 1) return hipSuccess;
+    if (dev != kMaxDevices - 1 && done[dev].load(std::memory_order_acquire)) return hipSuccess;
     e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (e == hipSuccess) done[dev] = true;
+    if (e == hipSuccess) done[dev].store(true, std::memory_order_release);
     return e;
 }
 

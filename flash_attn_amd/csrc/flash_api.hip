@@ -88,6 +88,12 @@ int validate(const flash_params* p, bool* empty)
 
 constexpr int kRowsPerGroup = 128;  // FwdCfg<D, 1>::BR
 
+// A window bound that can never cut (i' - j <= Nk - 1, j - i' <= Nq - 1 for the row index i' = i + Nk - Nq) is the same
+// as no bound; callers write "unbounded" as INT_MAX too, which the kernels' i' + right would overflow.  Everything
+// that looks at the window (launch arguments, kernel choice, split count) looks at these.
+inline int window_left_of(const flash_params* p) { return p->window_left >= p->Nk ? -1 : p->window_left; }
+inline int window_right_of(const flash_params* p) { return p->window_right >= p->Nq ? -1 : p->window_right; }
+
 void fill_args(const flash_params* p, int splits, fa::FwdArgs* a)
 {
     std::memset(a, 0, sizeof(*a));
@@ -111,10 +117,8 @@ void fill_args(const flash_params* p, int splits, fa::FwdArgs* a)
     a->Hk = p->H_kv > 0 ? p->H_kv : (p->H > 0 ? p->H : 1);
     a->kv_group = p->H > 0 ? p->H / a->Hk : 1;
     a->causal = p->is_causal ? 1 : 0;
-    // A bound that can never cut (i' - j <= Nk - 1, j - i' <= Nq - 1 for the row index i' = i + Nk - Nq) is the same
-    // as no bound; callers write "unbounded" as INT_MAX too, which the kernels' i' + right would overflow.
-    a->wl = p->window_left >= p->Nk ? -1 : p->window_left;
-    a->wr = p->window_right >= p->Nq ? -1 : p->window_right;
+    a->wl = window_left_of(p);
+    a->wr = window_right_of(p);
     a->alibi_left = (p->alibi_slopes && (a->causal || a->wr == 0)) ? 1 : 0;
     a->scale_log2 = p->softmax_scale * fa::kLog2e;
     a->drop_thr = flash_dropout_threshold(p->dropout_p);
@@ -162,6 +166,95 @@ long long tiled_groups(const flash_params* p, const fa::FwdArgs& a)
     return (long long)((a.Nq + rows - 1) / rows) * a.B * a.H * a.num_splits;
 }
 
+// Automatic split count of the tiled kernels (Nq > 1): the count with the lowest estimated time of split kernel +
+// combine.  The reference's rule (src/main.cu:391-422, called at :125) only asks how full the last round of thread
+// blocks over the SMs is, and only among counts with seq_len % (128 s) == 0, an artifact of its tiling (here the ranges
+// are whole 128-key blocks whatever s is).  Sweeps of explicit counts on 256 CUs showed what else decides:
+//  * work-groups i and i + 256 share a CU (the dispatcher deals them out round robin), so 320 work-groups take about as
+//    long as 512: the unit is the number k of work-groups on the fullest CU
+//    (B1 H8 Nq512 Nk32768 d128: 8 splits 87.6 us, 10: 100.5, 12: 91.9, 16: 84.2);
+//  * k work-groups of a CU run side by side and finish in less than k times the time of one (1.3x faster in all where
+//    the tiles come by LDS-DMA, 1.5-1.6x for the instances that are bound by load latency), but each pays a prologue
+//    and an epilogue, and each split its partial results: 8 B H Nq d bytes written and read back, at about 3.5 TB/s;
+//  * under a causal mask the launch takes as long as its heaviest work-group, the last row block's longest split, alone
+//    on its CU for most of its life: with few head slices splitting shortens exactly that
+//    (B1 H2 N16384 d64: 194 us unsplit, 124 us in 5 splits; B1 H16 N2048 d128 stays unsplit: 39 us against 44).
+// The estimate for s splits: k (a + b t) / rho + [s > 1] (c0 + s * partials), t = tiles of a work-group (the heaviest one
+// plus k - 1 average ones), b = microseconds per 64-key tile of a work-group alone on its CU, rho the gain of k side by
+// side.  Over 21 swept shapes the count it picks is within 5 % of the best measured one on 19 (the others: 5.4 % and
+// 15 %); the reference's rule with 256 CUs: 12 of 21, the worst 6.8 times slower than the best count.  Costs the host
+// up to 0.2 ms on very long sequences (a loop over row blocks per candidate count): callers on a tight loop pass an
+// explicit count, or the one flash_splitkv_resolve_splits returned for the shape.
+int auto_splits_tiled(const flash_params* p, int n_blocks)
+{
+    const int wl = window_left_of(p), wr = window_right_of(p);
+    const bool vec = (tiled_variant(p) & 1) != 0;
+    const bool pp = fa::fwd_uses_pingpong(p->d, vec, p->Nq, p->is_causal, wl, wr, (long long)p->B * p->H, p->kernel_hint);
+    const int rows = pp ? 256 : kRowsPerGroup;
+    const int Tr = (p->Nq + rows - 1) / rows;
+    const long long slices = (long long)p->B * p->H;
+    if (slices * Tr >= 4LL * kNumCU) return 1;  // (the reference's early exit: four rounds of work-groups as they are)
+    const int bucket = (p->d + 31) / 32;  // head-dim bucket of the kernel instance: 1 ... 4
+    // microseconds per tile of a lone work-group, by bucket; x 1.3 where the tiles are staged through registers
+    // (d % 8 == 0 but not the bucket's width), x 3.4 with element-wise loads (d % 8 != 0)
+    static const float kTile[5] = {0.0f, 0.5f, 0.72f, 0.88f, 1.0f};
+    const bool dma = vec && p->d == 32 * bucket;
+    const float b = pp ? 1.97f : kTile[bucket] * (dma ? 1.0f : vec ? 1.3f : 3.4f);
+    const float rho2 = pp ? 1.0f : dma ? 1.32f : vec ? 1.5f : 1.6f;
+    const float rho3 = (!pp && vec && p->d <= 64) ? rho2 * 1.12f : rho2;  // three places per CU up to d = 64
+    const float a = 6.0f, c0 = 5.0f;
+    const float partials = 8.0f * (float)slices * (float)p->Nq * (float)p->d / 3.5e6f;  // us per split
+    const int shift = p->Nk - p->Nq;
+    const bool masked = p->is_causal || wl >= 0 || wr >= 0;
+    int limit = FLASH_MAX_SPLITS;
+    if (n_blocks < limit) limit = n_blocks;
+    int best_s = 1, prev_per = -1;
+    float best_t = 0.0f;
+    for (int s = 1; s <= limit; ++s) {
+        const int per = (n_blocks + s - 1) / s;
+        if (per == prev_per) continue;  // the same ranges as s - 1 plus an empty split (src/main.cu:397-398)
+        prev_per = per;
+        const long long kps = (long long)per * FLASH_SPLIT_KEY_GRANULE;
+        // work-groups with a visible key, their tiles, and the tiles of the heaviest one
+        long long groups = 0, tiles = 0, tmax = 0;
+        const int m_end = masked ? Tr : 1;  // without a mask every row block sees every key
+        for (int m = 0; m < m_end; ++m) {
+            long long lo = 0, hi = p->Nk;  // visible keys of the row block: [lo, hi)
+            if (masked) {
+                const long long first = (long long)m * rows + shift;
+                const long long last = (long long)((m + 1) * rows < p->Nq ? (m + 1) * rows : p->Nq) - 1 + shift;
+                if (wl >= 0 && first - wl > lo) lo = first - wl;
+                if (p->is_causal && last + 1 < hi) hi = last + 1;
+                if (wr >= 0 && last + wr + 1 < hi) hi = last + wr + 1;
+                if (hi < 0) hi = 0;
+                if (lo > hi) lo = hi;
+            }
+            if (hi <= lo) continue;
+            const long long s_lo = lo / kps, s_hi = (hi - 1) / kps;
+            groups += s_hi - s_lo + 1;
+            tiles += (hi - lo + 63) / 64;
+            const long long longest = s_hi > s_lo ? kps : hi - lo;
+            if ((longest + 63) / 64 > tmax) tmax = (longest + 63) / 64;
+        }
+        if (!masked) {
+            groups *= Tr;
+            tiles *= Tr;
+        }
+        groups *= slices;
+        tiles *= slices;
+        if (groups == 0) return 1;
+        const long long k = (groups + kNumCU - 1) / kNumCU;
+        const float rho = k == 1 ? 1.0f : k == 2 ? rho2 : rho3;
+        float t = ((float)k * a + b * ((float)tmax + (float)(k - 1) * (float)tiles / (float)groups)) / rho;
+        if (s > 1) t += c0 + (float)s * partials;
+        if (s == 1 || t < best_t) {
+            best_t = t;
+            best_s = s;
+        }
+    }
+    return best_s;
+}
+
 int resolve_splits(const flash_params* p)
 {
     const int n_blocks = (p->Nk + FLASH_SPLIT_KEY_GRANULE - 1) / FLASH_SPLIT_KEY_GRANULE;
@@ -181,13 +274,7 @@ int resolve_splits(const flash_params* p)
         const int by_keys = n_blocks / 4;  // 512 keys per split
         s = (int)(want < by_keys ? want : by_keys);
     } else if (s <= 0) {
-        const bool vec = p->d % 8 == 0 && p->softmax_scale > 0.0f;
-        const int rows = fa::fwd_uses_pingpong(p->d, vec, p->Nq, p->is_causal, p->window_left, p->window_right,
-                                               (long long)p->B * p->H, p->kernel_hint) ? 256 : kRowsPerGroup;
-        const int Tr = (p->Nq + rows - 1) / rows;
-        // argument roles as in the reference's call (src/main.cu:125), with the CU count of the MI355X and the row
-        // blocks of the kernel that will run
-        s = flash_num_splits_heuristic(Tr * p->H * p->B, kNumCU, n_blocks, FLASH_MAX_SPLITS, n_blocks * FLASH_SPLIT_KEY_GRANULE);
+        s = auto_splits_tiled(p, n_blocks);
     }
     if (s > n_blocks) s = n_blocks;  // never more splits than key blocks
     if (s > FLASH_MAX_SPLITS) s = FLASH_MAX_SPLITS;
@@ -383,6 +470,15 @@ FLASH_EXPORT int flash_dropout_keep_mask(const flash_params* p, uint8_t* mask_ou
     if ((long long)p->B * p->H * p->Nq == 0 || p->Nk == 0) return FLASH_OK;
     return record_hip(fa::launch_keep_mask(mask_out, p->B, p->H, p->Nq, p->Nk, flash_dropout_threshold(p->dropout_p),
                                            p->seed, p->offset, static_cast<hipStream_t>(stream)));
+}
+
+FLASH_EXPORT void flash_params_init(flash_params* p)
+{
+    if (!p) return;
+    std::memset(p, 0, sizeof(*p));
+    p->window_left = -1;
+    p->window_right = -1;
+    p->num_splits = 1;
 }
 
 FLASH_EXPORT size_t flash_params_size(void) { return sizeof(flash_params); }

@@ -127,7 +127,8 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     int bh, rest;
     {
         const int per_chunk = a.slice_chunk * a.Tr * a.num_splits;
-        const int ch = blockIdx.x / per_chunk, w = blockIdx.x % per_chunk;
+        const int pos = work_position(blockIdx.x, a.snake_end);
+        const int ch = pos / per_chunk, w = pos % per_chunk;
         bh = ch * a.slice_chunk + w % a.slice_chunk;
         rest = w / a.slice_chunk;
     }
@@ -369,7 +370,12 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                         // folded in, from the per-register bias constants, which stay where they are
                         if constexpr (folded) {
                             // written out: the compiler only knows the form whose result overwrites the addend and would
-                            // copy the sixteen constants for every tile
+                            // copy the sixteen constants for every tile.  Hazards of an MFMA the compiler cannot see as
+                            // one: its operands are ready (the asm's inputs: af comes with the wait for its LDS read,
+                            // qf and calib were written long before); its result is next read as the addend of the
+                            // second k-step's MFMA on the same registers, a dependency the hardware interlocks -- hence
+                            // at least two k-steps -- and by VALU code only after that one.
+                            static_assert(!folded || KS >= 2, "the score accumulator is first read by a following MFMA");
                             asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(s[kb][nb]) : "v"(af), "v"(qf[nb][ks]), "v"(calib));
                         } else {
                             const v16f z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -799,12 +805,14 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
 {
     using C = FwdCfg<D, NB>;
     auto kern = fwd_kernel<D, NB, VAR>;
-    static bool attr_done[kMaxDevices] = {};  // per instantiation and device
+    static DeviceFlags attr_done;  // per instantiation and device
     constexpr int smem = C::SMEM_DMA > C::SMEM ? C::SMEM_DMA : C::SMEM;  // (equal: both paths use two stages)
     if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, attr_done); e != hipSuccess) return e;
     const long long groups = (long long)a.Tr * a.B * a.H * a.num_splits;
     FwdArgs b = a;
-    b.slice_chunk = slice_chunk_for(a.B * a.H, a.Tr * a.num_splits, (NB == 1 && D <= 64 && (VAR & kVarVec) != 0 ? 3 : 2) * kNumCus);
+    constexpr int kResident = (NB == 1 && D <= 64 && (VAR & kVarVec) != 0 ? 3 : 2) * kNumCus;
+    b.slice_chunk = slice_chunk_for(a.B * a.H, a.Tr * a.num_splits, kResident);
+    b.snake_end = snake_end_for(groups, kResident);
     return launch_kernel(kern, dim3((unsigned)groups), dim3(256), smem, st, b);
 }
 

@@ -91,7 +91,8 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     int bh, rest;
     {
         const int per_chunk = a.slice_chunk * a.Tr * a.num_splits;
-        const int ch = blockIdx.x / per_chunk, w = blockIdx.x % per_chunk;
+        const int pos = work_position(blockIdx.x, a.snake_end);  // (one work-group per CU: the identity)
+        const int ch = pos / per_chunk, w = pos % per_chunk;
         bh = ch * a.slice_chunk + w % a.slice_chunk;
         rest = w / a.slice_chunk;
     }
@@ -638,12 +639,13 @@ inline hipError_t launch_fwd_pp_instance(const FwdArgs& a, hipStream_t st)
 {
     using C = PPCfg<D>;
     auto kern = fwd_pp_kernel<D, VAR>;
-    static bool attr_done[kMaxDevices] = {};  // per instantiation and device
+    static DeviceFlags attr_done;  // per instantiation and device
     if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), C::SMEM, attr_done); e != hipSuccess) return e;
     FwdArgs b = a;
     b.Tr = (a.Nq + C::BR - 1) / C::BR;
     const long long groups = (long long)b.Tr * a.B * a.H * a.num_splits;
     b.slice_chunk = slice_chunk_for(a.B * a.H, b.Tr * a.num_splits, kNumCus);  // one work-group per CU at a time
+    b.snake_end = snake_end_for(groups, kNumCus);
     return launch_kernel(kern, dim3((unsigned)groups), dim3(512), C::SMEM, st, b);
 }
 

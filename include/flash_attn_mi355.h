@@ -53,6 +53,11 @@ enum {
  *   dropout_prob, seed, states dropout_p, seed, offset   counter-based Philox4x32-10 instead of curand states
  *   split_num                  num_splits          (<= 0: chosen by the library, see flash_forward_splitkv)
  * Row index used by masks and bias is i + (Nk - Nq), which is i whenever Nq == Nk (all the reference can express).
+ *
+ * EVERY field is read by the library: start from flash_params_init() (or from an all-zero struct with window_left =
+ * window_right = -1) and set what the call needs.  A field left uninitialised is not detected -- a stray kernel_hint is
+ * rejected with FLASH_EINVAL, a stray debug-output pointer is written through.  Fields are only ever appended to the
+ * struct; flash_params_size() lets a caller built against another header notice before its first call.
  */
 typedef struct flash_params {
     const void *Q;
@@ -162,6 +167,13 @@ int flash_dropout_keep_mask(const flash_params *p, uint8_t *mask_out, void *stre
  * up of output word f >> 1), and element (i, j) is kept iff field 4*((j >> 3) & 1) + (j & 3) >= threshold.  Kept
  * probabilities are scaled by 1/(1 - dropout_p); the row sum of the softmax is taken before the drop. */
 uint32_t flash_dropout_threshold(float dropout_p);
+
+/* Defaults for every field: all pointers NULL, all sizes 0, no mask (is_causal 0, window_left = window_right = -1), no
+ * bias, no dropout, num_splits 1 (unsplit), H_kv 0 (= H), kernel_hint 0, no debug outputs.  softmax_scale stays 0: the
+ * caller sets it (the reference uses 1/sqrt(d), src/main.cu:112).  The reference fills its struct field by field and
+ * leaves dropout_prob, states, split_num, O_tmp, L and M uninitialised on the paths that do not use them
+ * (src/main.cu:109-123); this helper is what a binding calls first instead.  NULL is ignored. */
+void flash_params_init(flash_params *p);
 
 /* sizeof(flash_params) of the header the library was built with.  A caller compiled against another version of the
  * header would hand over a struct of another size (fields are only ever appended): compare before the first call. */

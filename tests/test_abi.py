@@ -130,10 +130,32 @@ def test_split_resolution_and_workspace(fa):
     assert fa.resolve_splits(1, 1, 1, 300, 64, 16) == 3
     assert fa.resolve_splits(1, 1, 128, 128, 64, 8) == 1
     assert fa.workspace_bytes(1, 1, 128, 128, 64, 8) == (0, 0)
-    # heuristic (num_splits <= 0) with 256 CUs: the reference's checked-in shape B=1,H=8,N=1021 splits 4 ways,
-    # the prefill benchmark shapes stay unsplit
+    # automatic choice (num_splits <= 0) for Nq > 1: the count with the lowest estimated time (work-groups on the fullest
+    # CU, prologue / epilogue per work-group, partial results per split).  The reference's checked-in shape
+    # B=1,H=8,N=1021 splits 4 ways (64 row blocks -> 256 work-groups), twice that batch as well (its element-wise loads
+    # gain from a second work-group per CU), the prefill benchmark shapes stay unsplit
     assert fa.resolve_splits(1, 8, 1021, 1021, 31, 0) == 4
+    assert fa.resolve_splits(2, 8, 1021, 1021, 31, 0) == 4
     assert fa.resolve_splits(4, 16, 2048, 2048, 128, 0) == 1
+    assert fa.resolve_splits(4, 16, 2048, 2048, 128, 0, causal=True) == 1
+    assert fa.resolve_splits(8, 32, 1000, 1000, 96, 0, causal=True) == 1
+    # long keys, few rows: one work-group per CU; two where a split stays long enough to pay for them
+    assert fa.resolve_splits(1, 8, 512, 32768, 128, 0) == 16
+    assert fa.resolve_splits(1, 32, 128, 16384, 128, 0, causal=True) == 8
+    assert fa.resolve_splits(1, 16, 256, 8192, 64, 0) == 8
+    assert fa.resolve_splits(1, 4, 1024, 65536, 64, 0) == 16
+    assert fa.resolve_splits(1, 40, 128, 8192, 128, 0) == 6      # 240 work-groups, not five rounds of short ones
+    assert fa.resolve_splits(2, 4, 300, 20000, 96, 0) == 10
+    # 10 key blocks, 52 work-groups: 4 splits of 3 blocks fill 208 of 256 CUs (the reference's rule only looks at counts
+    # with 1280 % (128 s) == 0 and would take 10 splits of one block)
+    assert fa.resolve_splits(1, 52, 100, 1280, 64, 0) == 4
+    assert fa.num_splits_heuristic(52, 256, 10, 128, 1280) == 10
+    # causal with one work-group per CU at most: split along the keys when the heaviest row block is long enough to
+    # pay for the partial results
+    assert fa.resolve_splits(1, 16, 2048, 2048, 128, 0, causal=True) == 1
+    assert fa.resolve_splits(1, 2, 16384, 16384, 64, 0, causal=True) == 5
+    # a narrow window leaves a row block two or three key blocks: nothing to split
+    assert fa.resolve_splits(1, 4, 4096, 4096, 64, 0, window=(256, 0)) == 1
     # one query row (decode, bandwidth-bound): about 32 work-groups per CU, 512 keys or more per split
     assert fa.resolve_splits(16, 32, 1, 16384, 128, 0) == 16
     assert fa.resolve_splits(1, 32, 1, 16384, 128, 0) == 32

@@ -185,6 +185,49 @@ def test_general_splitkv_matches_unsplit(fa, oracle, S):
             assert np.abs(op - Ot).max() <= 2e-3
 
 
+@pytest.mark.parametrize("B,H,Nq,Nk,d,causal,want", [
+    (1, 8, 512, 32768, 128, False, 16),   # long keys, small batch: two work-groups per CU
+    (1, 32, 128, 16384, 128, True, 8),    # causal with Nq < Nk: every split holds visible keys
+    (2, 8, 1021, 1021, 31, False, 4),     # twice the reference's checked-in run (src/main.cu:39-49)
+    (1, 2, 8192, 8192, 64, True, None),   # causal, one work-group per CU at most: split for the heaviest row block
+    (1, 40, 128, 8192, 128, False, 6),
+])
+def test_automatic_split_count_shapes(fa, oracle, B, H, Nq, Nk, d, causal, want):
+    """num_splits <= 0 for Nq > 1: the library's own count (more than one on these shapes) gives the unsplit result; the
+    first and the last head slice are checked against the oracle."""
+    q, k, v = _qkv(B, H, Nq, Nk, d, seed=B + H + d)
+    S = fa.resolve_splits(B, H, Nq, Nk, d, 0, causal=causal)
+    assert S > 1 and (want is None or S == want)
+    o, lse, ws = fa.flash_forward_splitkv(q, k, v, num_splits=0, causal=causal, return_partials=True)
+    assert ws[0].shape == (B, H, S, Nq, d)
+    o1, lse1 = fa.flash_forward(q, k, v, causal=causal)
+    assert (o.float() - o1.float()).abs().max().item() <= 2e-3
+    assert (lse - lse1).abs().max().item() <= 1e-4
+    for b, h in ((0, 0), (B - 1, H - 1)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        O, L = oracle_forward_batched(oracle, q[sl], k[sl], v[sl], causal=causal)
+        check_o_lse(o[sl], lse[sl], O, L, f"auto split S={S} slice ({b},{h})")
+
+
+@pytest.mark.parametrize("B,H,N,d", [(1, 32, 2048, 128), (1, 48, 2048, 64), (1, 30, 1200, 96), (3, 33, 700, 128)])
+def test_resident_work_groups_in_snake_order(fa, oracle, B, H, N, d):
+    """Launches whose work-groups all sit on the GPU at once (here 350-770 of them at two or three per CU) run every
+    second block of 256 work-groups in reverse order; every (slice, row block) must still be served exactly once --
+    also where the resident part ends inside a block of 256 or is no multiple of 8."""
+    import torch
+    q, k, v = _qkv(B, H, N, N, d, seed=N + d)
+    o, lse = fa.flash_forward(q, k, v, causal=True, kernel_hint=fa.KERNEL_4WAVE)
+    for b, h in ((0, 0), (B - 1, H - 1), (B // 2, H // 2), (0, H - 1)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        O, L = oracle_forward_batched(oracle, q[sl], k[sl], v[sl], causal=True)
+        check_o_lse(o[sl], lse[sl], O, L, f"slice ({b},{h})")
+    # every row written: compare all slices with a launch that is far beyond the resident part (chunks of slices)
+    o2, lse2 = fa.flash_forward(torch.cat([q] * 4), torch.cat([k] * 4), torch.cat([v] * 4), causal=True,
+                                kernel_hint=fa.KERNEL_4WAVE)
+    for r in range(4):
+        assert torch.equal(o2[r * B:(r + 1) * B], o) and torch.equal(lse2[r * B:(r + 1) * B], lse)
+
+
 def test_splitkv_heuristic_and_decode_variants(fa, oracle):
     # num_splits <= 0: the library's heuristic (4 splits for this shape on 256 CUs)
     q, k, v = _qkv(1, 8, 1021, 1021, 32, seed=3)

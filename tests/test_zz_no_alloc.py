@@ -54,21 +54,77 @@ def test_static_scratch_matches_workspace_entry_point(fa, oracle, first, second)
 
 
 def test_static_scratch_rejects_what_does_not_fit(fa):
-    """B=64, H=64, 128 splits of one query row at d=128 need 270 MB of partials: an error code, nothing launched (K and V
-    point at a buffer far smaller than the shape says, which a launch would overrun)."""
+    """B=1, H=16, 2048 rows, 4 splits at d=128 need 64 MiB of partials, twice the scratch: an error code and nothing
+    launched.  Every buffer has the size the shape says, so that a regression of the check shows as a wrong return code
+    or a changed output, not as a kernel reading out of bounds."""
     import torch
 
-    q = torch.zeros((64, 64, 1, 128), dtype=torch.float16, device="cuda")
-    kv = torch.zeros(4096, dtype=torch.float16, device="cuda")
-    o = torch.full_like(q, 7.0)
-    lse = torch.zeros((64, 64, 1), dtype=torch.float32, device="cuda")
-    p = fa.FlashParams()
-    p.Q, p.K, p.V, p.O, p.LSE = q.data_ptr(), kv.data_ptr(), kv.data_ptr(), o.data_ptr(), lse.data_ptr()
-    p.B, p.H, p.Nq, p.Nk, p.d = 64, 64, 1, 16384, 128
-    p.softmax_scale = 0.1
-    p.window_left = p.window_right = -1
-    p.num_splits = 128
+    B, H, Nq, Nk, d, S = 1, 16, 2048, 512, 128, 4
+    q = randn_f16_gpu((B, H, Nq, d), 61)
+    k = randn_f16_gpu((B, H, Nk, d), 62)
+    v = randn_f16_gpu((B, H, Nk, d), 63)
+    assert sum(fa.workspace_bytes(B, H, Nq, Nk, d, S)) > fa.FLASH_STATIC_SCRATCH_BYTES
+    o = torch.full((B, H, Nq, d), 7.0, dtype=torch.float16, device="cuda")
+    lse = torch.full((B, H, Nq), 7.0, dtype=torch.float32, device="cuda")
+    from flash_attn_amd import binding
+    p = binding.make_params(q, k, v, o, lse, None, False, (-1, -1), None, 0.0, 0, 0, S)
     rc = fa.lib().flash_forward_splitkv_static(C.byref(p), None)
     assert rc == -8 and b"scratch" in fa.lib().flash_strerror(rc)
     torch.cuda.synchronize()
-    assert bool((o == 7.0).all())
+    assert bool((o == 7.0).all()) and bool((lse == 7.0).all())
+    # one split fewer rows: 32 MiB + 256 KiB still does not fit; half the rows do
+    p.Nq = 1024
+    assert fa.lib().flash_forward_splitkv_static(C.byref(p), None) == -8
+    p.Nq = 1000
+    assert fa.lib().flash_forward_splitkv_static(C.byref(p), None) == 0
+    torch.cuda.synchronize()
+    # (the static call read rows 0..999 of every head slice at the stride of 1000 rows: compare on a contiguous copy)
+    qc = q.reshape(-1)[:B * H * 1000 * d].view(B, H, 1000, d)
+    o_c, lse_c = fa.flash_forward_splitkv(qc.contiguous(), k, v, num_splits=S)
+    assert torch.equal(o.reshape(-1)[:B * H * 1000 * d].view(B, H, 1000, d), o_c)
+    assert torch.equal(lse.reshape(-1)[:B * H * 1000].view(B, H, 1000), lse_c)
+
+
+def test_static_entry_point_allocates_nothing_and_replays_from_a_graph(fa):
+    """The two promises beyond bit-identical results: no device memory is allocated or freed by the call (the free
+    memory the runtime reports and the bytes PyTorch holds are the same before and after), and the call can be captured
+    into a HIP graph -- three replays with new inputs in between, each compared with an eager call of the workspace
+    entry point."""
+    import torch
+    from flash_attn_amd import binding
+
+    B, H, Hk, Nq, Nk, d, S = 2, 8, 8, 1, 6000, 128, 6
+    q = randn_f16_gpu((B, H, Nq, d), 71)
+    k = randn_f16_gpu((B, Hk, Nk, d), 72)
+    v = randn_f16_gpu((B, Hk, Nk, d), 73)
+    o = torch.empty((B, H, Nq, d), dtype=torch.float16, device="cuda")
+    lse = torch.empty((B, H, Nq), dtype=torch.float32, device="cuda")
+    p = binding.make_params(q, k, v, o, lse, None, False, (-1, -1), None, 0.0, 0, 0, S)
+    L = fa.lib()
+
+    def call():
+        rc = L.flash_forward_splitkv_static(C.byref(p), C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, L.flash_strerror(rc)
+
+    call()  # first call on the device and of this shape class: symbol look-up, kernel attributes
+    torch.cuda.synchronize()
+    free0, held0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0 and torch.cuda.memory_allocated() == held0
+
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        call()
+    for rep in range(3):
+        q.copy_(randn_f16_gpu((B, H, Nq, d), 300 + rep))
+        k.copy_(randn_f16_gpu((B, Hk, Nk, d), 400 + rep))
+        o.zero_()
+        lse.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        o_e, lse_e = fa.flash_forward_splitkv(q, k, v, num_splits=S)  # eager, workspace of its own
+        torch.cuda.synchronize()
+        assert torch.equal(o, o_e) and torch.equal(lse, lse_e), f"replay {rep} differs from the eager call"
