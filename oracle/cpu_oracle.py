@@ -10,7 +10,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+# FLASH_ORACLE_LIB: another build of the same source (the sanitizer build of tests/test_sanitizers.py)
+_LIB_PATH = os.environ.get("FLASH_ORACLE_LIB") or os.path.join(_HERE, "liboracle.so")
 _REF_PATH = os.path.join(_HERE, "_ref", "libref_cpu.so")
 
 _f32p = C.POINTER(C.c_float)
@@ -67,6 +68,10 @@ def lib():
         L.oracle_dropout_keep_mask.restype = None
         L.oracle_dropout_keep_mask.argtypes = [C.c_uint64, C.c_uint64, C.c_float] + [C.c_int] * 4 + [_u8p, C.c_int]
         L.oracle_max_threads.restype = C.c_int
+        L.oracle_f32_to_f16.restype = None
+        L.oracle_f32_to_f16.argtypes = [_f32p, C.c_void_p, C.c_uint64]
+        L.oracle_fill_normal_f16.restype = None
+        L.oracle_fill_normal_f16.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int]
         _lib = L
     return _lib
 
@@ -170,6 +175,23 @@ def philox4x32_10(ctr, key):
     o = (C.c_uint32 * 4)()
     lib().oracle_philox4x32_10(c, k, o)
     return [int(x) for x in o]
+
+
+def normal_f16(shape, seed, first=0, nthreads=None):
+    """RN_fp16(N(0,1)) of the portable generator: element e of the flattened array is a function of (seed, first + e)."""
+    n = int(np.prod(shape, dtype=np.int64))
+    out = np.empty(n, dtype=np.uint16)
+    lib().oracle_fill_normal_f16(out.ctypes.data_as(C.c_void_p), int(first), n, int(seed),
+                                 int(nthreads or default_threads()))
+    return out.view(np.float16).reshape(shape)
+
+
+def f32_to_f16_bits(x):
+    """fp16 bit patterns of the generator's own round-to-nearest-even conversion (for tests)."""
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    out = np.empty(x.size, dtype=np.uint16)
+    lib().oracle_f32_to_f16(_fp(x), out.ctypes.data_as(C.c_void_p), x.size)
+    return out
 
 
 def dropout_threshold(p):

@@ -26,6 +26,7 @@ int oracle_attention_forward(const float* Q, const float* K, const float* V, int
                              float scale, int causal, int window_left, int window_right, const float* slopes,
                              const uint8_t* keep_mask, float p_drop, float* O, float* LSE, int nthreads);
 int oracle_max_threads(void);
+void oracle_fill_normal_f16(uint16_t* out, uint64_t first, uint64_t count, uint64_t seed, int nthreads);
 }
 
 namespace {
@@ -40,6 +41,8 @@ struct Options {
     float tol = 0.06f;
     long long max_print = 20;
     std::string fill = "reference";
+    unsigned long long seed = 1;  // --fill normal: Q from seed, K from seed + 1, V from seed + 2
+    std::string dump;             // --dump-inputs
 };
 
 void usage(const char* argv0)
@@ -53,7 +56,10 @@ void usage(const char* argv0)
         "  --dropout P                                  dropout probability (disables the check, as the reference does)\n"
         "  --splits S                                   key splits: 0 = heuristic (default), S > 0 explicit\n"
         "  --iters K --warmup W                         timed / untimed launches (default 1000 / 1)\n"
-        "  --fill reference|normal                      U(0,10) with engine seed 26 (default) or N(0,1), seed 26\n"
+        "  --fill reference|normal                      U(0,10) with engine seed 26 (default), or RN_fp16(N(0,1)) from the\n"
+        "                                               portable counter-based generator (the test harness's inputs)\n"
+        "  --seed S                                     --fill normal: Q from seed S, K from S + 1, V from S + 2 (default 1)\n"
+        "  --dump-inputs FILE                           write the fp16 bits of Q, K, V to FILE and exit (no GPU needed)\n"
         "  --tol T                                      relative error bound of the check (default 0.06)\n"
         "  --max-print M                                print at most M mismatches (default 20, -1: all)\n"
         "  --no-verify                                  skip the CPU forward and the check\n",
@@ -83,6 +89,8 @@ bool parse(int argc, char** argv, Options* o)
         else if (a == "--iters") o->iters = std::atoi(next("--iters"));
         else if (a == "--warmup") o->warmup = std::atoi(next("--warmup"));
         else if (a == "--fill") o->fill = next("--fill");
+        else if (a == "--seed") o->seed = std::strtoull(next("--seed"), nullptr, 10);
+        else if (a == "--dump-inputs") o->dump = next("--dump-inputs");
         else if (a == "--tol") o->tol = (float)std::atof(next("--tol"));
         else if (a == "--max-print") o->max_print = std::atoll(next("--max-print"));
         else if (a == "--no-verify") o->verify = false;
@@ -135,29 +143,49 @@ int main(int argc, char** argv)
     const int B = opt.batch, H = opt.heads, N = opt.seq, d = opt.head_dim;
     const size_t n = (size_t)B * H * N * d;
 
+    // ---- host data: the reference's fill (order of src/main.cu:91-103), or the portable N(0,1) generator
+    std::vector<float> Q(n), K(n), V(n), O(n, 0.0f), O_host(n);
+    std::vector<_Float16> Qh(n), Kh(n), Vh(n), Oh(n);
+    if (opt.fill == "reference") {
+        std::default_random_engine generator(26);
+        std::uniform_real_distribution<float> uniform(0.0f, 10.0f);
+        for (size_t i = 0; i < n; i++) {
+            Q[i] = uniform(generator);
+            K[i] = uniform(generator);
+            V[i] = uniform(generator);
+            Qh[i] = (_Float16)Q[i];
+            Kh[i] = (_Float16)K[i];
+            Vh[i] = (_Float16)V[i];
+        }
+    } else {
+        static_assert(sizeof(_Float16) == sizeof(uint16_t), "fp16 storage");
+        const int th = oracle_max_threads();
+        oracle_fill_normal_f16(reinterpret_cast<uint16_t*>(Qh.data()), 0, n, opt.seed, th);
+        oracle_fill_normal_f16(reinterpret_cast<uint16_t*>(Kh.data()), 0, n, opt.seed + 1, th);
+        oracle_fill_normal_f16(reinterpret_cast<uint16_t*>(Vh.data()), 0, n, opt.seed + 2, th);
+        for (size_t i = 0; i < n; i++) {  // the CPU forward sees the fp16 values, widened
+            Q[i] = (float)Qh[i];
+            K[i] = (float)Kh[i];
+            V[i] = (float)Vh[i];
+        }
+    }
+    if (!opt.dump.empty()) {
+        FILE* f = std::fopen(opt.dump.c_str(), "wb");
+        if (!f) {
+            std::perror(opt.dump.c_str());
+            return 1;
+        }
+        const bool ok = std::fwrite(Qh.data(), 2, n, f) == n && std::fwrite(Kh.data(), 2, n, f) == n &&
+                        std::fwrite(Vh.data(), 2, n, f) == n;
+        return std::fclose(f) == 0 && ok ? 0 : 1;
+    }
+
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) {
         std::fprintf(stderr, "%s\n", flash_strerror(FLASH_ENODEVICE));
         return 1;
     }
 
-    // ---- host data (fill order of src/main.cu:91-103)
-    std::vector<float> Q(n), K(n), V(n), O(n, 0.0f), O_host(n);
-    std::vector<_Float16> Qh(n), Kh(n), Vh(n), Oh(n);
-    {
-        std::default_random_engine generator(26);
-        std::uniform_real_distribution<float> uniform(0.0f, 10.0f);
-        std::normal_distribution<float> normal(0.0f, 1.0f);
-        const bool ref = opt.fill == "reference";
-        for (size_t i = 0; i < n; i++) {
-            Q[i] = ref ? uniform(generator) : normal(generator);
-            K[i] = ref ? uniform(generator) : normal(generator);
-            V[i] = ref ? uniform(generator) : normal(generator);
-            Qh[i] = (_Float16)Q[i];
-            Kh[i] = (_Float16)K[i];
-            Vh[i] = (_Float16)V[i];
-        }
-    }
     std::vector<float> slopes;
     float* slopes_dev = nullptr;
     if (opt.alibi) {
@@ -184,7 +212,7 @@ int main(int argc, char** argv)
         return 2;
     }
     flash_params p;
-    std::memset(&p, 0, sizeof(p));
+    flash_params_init(&p);
     p.Q = Qd;
     p.K = Kd;
     p.V = Vd;

@@ -35,6 +35,33 @@ def test_driver_is_not_older_than_the_header():
     assert r.returncode == 0, "tests/driver/flash_driver is stale: run `make -C tests/driver`"
 
 
+def test_driver_and_python_harness_draw_the_same_normal_inputs(tmp_path):
+    """`--fill normal --seed S` fills Q, K, V from the portable generator with seeds S, S + 1, S + 2: the same fp16 bits
+    as tests/helpers.py draws for those seeds (no GPU needed: --dump-inputs stops before the first HIP call)."""
+    import numpy as np
+    import sys
+
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from oracle import cpu_oracle
+
+    B, H, N, d = 2, 3, 37, 31
+    n = B * H * N * d
+    for seed in (1, 77):
+        f = tmp_path / f"inputs_{seed}.bin"
+        r = _run("--fill", "normal", "--seed", str(seed), "--batch", str(B), "--heads", str(H), "--seq", str(N),
+                 "--head-dim", str(d), "--dump-inputs", str(f))
+        assert r.returncode == 0, r.stderr
+        bits = np.fromfile(f, dtype=np.uint16)
+        assert bits.size == 3 * n
+        for t in range(3):
+            want = cpu_oracle.normal_f16((B, H, N, d), seed + t).view(np.uint16).ravel()
+            assert np.array_equal(bits[t * n:(t + 1) * n], want), (seed, t)
+    # the harness's device tensors are copies of exactly these arrays
+    import inspect
+    import helpers
+    assert "cpu_oracle.normal_f16" in inspect.getsource(helpers.randn_f16_gpu)
+
+
 def test_mfma_rate_probe_is_built():
     assert os.path.exists(os.path.join(ROOT, "tests", "driver", "mfma_rate")), "run `make -C tests/driver`"
 

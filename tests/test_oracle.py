@@ -202,6 +202,74 @@ def test_philox_against_independent_python(oracle):
         assert oracle.philox4x32_10(ctr, key) == py_philox(ctr, key)
 
 
+# ------------------------------------------------------------------------------ portable N(0,1) input generator
+def test_normal_generator_known_bits_and_definition(oracle):
+    """First 16 values of seed 1 as committed bit patterns, and the definition restated independently (Python Philox,
+    numpy float64 Box-Muller, numpy's own fp16 rounding) for several seeds and positions."""
+    want = [47206, 44509, 47317, 16233, 16322, 48526, 48225, 12740, 11490, 41946, 16407, 47885, 15396, 13524, 9249, 44365]
+    assert oracle.normal_f16((16,), 1).view(np.uint16).tolist() == want
+
+    def py_philox(ctr, key):
+        c, k = list(ctr), list(key)
+        for _ in range(10):
+            p0, p1 = 0xD2511F53 * c[0], 0xCD9E8D57 * c[2]
+            c = [((p1 >> 32) ^ c[1] ^ k[0]) & 0xFFFFFFFF, p1 & 0xFFFFFFFF, ((p0 >> 32) ^ c[3] ^ k[1]) & 0xFFFFFFFF,
+                 p0 & 0xFFFFFFFF]
+            k = [(k[0] + 0x9E3779B9) & 0xFFFFFFFF, (k[1] + 0xBB67AE85) & 0xFFFFFFFF]
+        return c
+
+    for seed, first in ((1, 0), (3, 4000), (0xDEADBEEF12345, 1 << 33), (2, 7)):
+        got = oracle.normal_f16((24,), seed, first=first)
+        z = []
+        for c in range(first // 4, (first + 24 + 3) // 4):
+            w = py_philox([c & 0xFFFFFFFF, c >> 32, 0x4E4F524D, 0], [seed & 0xFFFFFFFF, seed >> 32])
+            for a, b in ((w[0], w[1]), (w[2], w[3])):
+                r = np.sqrt(-2.0 * np.log((a + 1.0) / 4294967296.0))
+                ang = 2.0 * np.pi * (b / 4294967296.0)
+                z += [r * np.cos(ang), r * np.sin(ang)]
+        z = np.array(z[first % 4:first % 4 + 24])
+        assert np.array_equal(got.view(np.uint16), z.astype(np.float32).astype(np.float16).view(np.uint16)), (seed, first)
+
+
+def test_normal_generator_is_a_function_of_seed_and_position(oracle):
+    a = oracle.normal_f16((5000,), 9, nthreads=1)
+    assert np.array_equal(a.view(np.uint16), oracle.normal_f16((5000,), 9, nthreads=7).view(np.uint16))
+    for first in (1, 2, 3, 4, 1001, 4093):
+        part = oracle.normal_f16((700,), 9, first=first)
+        assert np.array_equal(part.view(np.uint16), a[first:first + 700].view(np.uint16)), first
+    assert not np.array_equal(a.view(np.uint16), oracle.normal_f16((5000,), 10).view(np.uint16))
+    assert oracle.normal_f16((2, 3, 5, 7), 4).shape == (2, 3, 5, 7)
+
+
+def test_normal_generator_moments_and_distribution(oracle):
+    from scipy import stats
+
+    x = oracle.normal_f16((1 << 20,), 5).astype(np.float64)
+    assert abs(x.mean()) < 4e-3 and abs(x.std() - 1.0) < 3e-3
+    assert abs(stats.skew(x)) < 1e-2 and abs(stats.kurtosis(x)) < 2e-2
+    assert stats.kstest(x[:200000], "norm").pvalue > 1e-3
+    # neighbours and the two members of a Box-Muller pair are uncorrelated
+    for lag in (1, 2, 3, 4):
+        assert abs(np.corrcoef(x[:-lag], x[lag:])[0, 1]) < 5e-3
+
+
+def test_generator_fp16_rounding_is_ieee_nearest_even(oracle):
+    rng = np.random.default_rng(11)
+    x = np.concatenate([
+        rng.standard_normal(200000).astype(np.float32) * np.float32(4),
+        (rng.standard_normal(50000) * 1e-5).astype(np.float32),           # subnormal halves
+        (rng.standard_normal(20000) * 1e-8).astype(np.float32),           # below the smallest subnormal
+        np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 70000.0, -1e9, np.inf, -np.inf, 2.0 ** -24, 2.0 ** -25,
+                  1.5 * 2.0 ** -25, 2.0 ** -14, 2.0 ** -14 - 2.0 ** -25, 1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11,
+                  2047.5, 2048.5, 0.999755859375 + 2.0 ** -13], dtype=np.float32)])
+    # every halfway case between neighbouring halves around 1 and 1024
+    h = np.arange(0x3BF0, 0x3C10, dtype=np.uint16).view(np.float16).astype(np.float32)
+    x = np.concatenate([x, (h[:-1] + h[1:]) / np.float32(2), np.float32(1024) * (h[:-1] + h[1:]) / np.float32(2)])
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(oracle.f32_to_f16_bits(x), want)
+
+
 def test_dropout_threshold_and_mask_layout(oracle):
     assert oracle.dropout_threshold(0.0) == 0
     assert oracle.dropout_threshold(0.5) == 2 ** 15
