@@ -53,6 +53,7 @@ struct FwdArgs {
     int alibi_left;      // ALiBi and no visible key lies right of its row (causal, or right window 0)
     int slice_chunk;     // head slices per chunk of the work-group order (set by the kernel's launcher)
     int snake_end;       // work-groups below this index sit on the GPU together; odd 256-blocks of them run reversed (launcher)
+    int group_xcd;       // > 1: query heads per K/V head, and the slice order keeps the heads of a K/V head on one XCD (launcher)
 
     // index of the K/V slice [Nk,d] read by query slice bh = b * H + h
     __device__ __forceinline__ int kv_slice(int bh) const { return (bh / H) * Hk + (bh % H) / kv_group; }
@@ -77,6 +78,21 @@ __device__ __forceinline__ int work_position(int block, int snake_end)
         return base + ((size >> 3) - 1 - (pos >> 3)) * 8 + (pos & 7);
     }
     return block;
+}
+
+// Head slice of position `local` in a chunk of the slice order.  Position p runs on XCD p % 8 (slices vary fastest over
+// the work-groups).  With grouped K/V heads the G = group_xcd query heads of a K/V head are G consecutive slices and would
+// land on G different XCDs, each pulling the same K and V into its own L2 (measured on B4 H32 H_kv4 N4096 d128 causal:
+// 3.7 times the K/V/Q bytes fetched).  Instead position (x, y) = (p % 8, p / 8) takes query head y % G of K/V slice
+// 8 (y / G) + x: the heads of a K/V head share an XCD and follow each other there.  A bijection on chunks whose size is
+// a multiple of 8 G (the launcher sets group_xcd only then).
+__device__ __forceinline__ int slice_of_position(int local, int group_xcd)
+{
+    if (group_xcd > 1) {
+        const int x = local & 7, y = local >> 3;
+        return ((y / group_xcd) * 8 + x) * group_xcd + y % group_xcd;
+    }
+    return local;
 }
 
 // snake_end for a launch of `groups` work-groups with `resident` places on the GPU

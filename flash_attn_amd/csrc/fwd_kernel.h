@@ -129,7 +129,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
         const int per_chunk = a.slice_chunk * a.Tr * a.num_splits;
         const int pos = work_position(blockIdx.x, a.snake_end);
         const int ch = pos / per_chunk, w = pos % per_chunk;
-        bh = ch * a.slice_chunk + w % a.slice_chunk;
+        bh = ch * a.slice_chunk + slice_of_position(w % a.slice_chunk, a.group_xcd);
         rest = w / a.slice_chunk;
     }
     const int split = rest % a.num_splits;
@@ -791,13 +791,27 @@ bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr, long
 // slices in one chunk: causal B16 H32 N1024 d128 +5 %, B8 H32 N2048 d64 +4 %, B8 H32 N4096 d128 (8-wave kernel) +16 %;
 // once or four times the resident work-groups per chunk instead of twice: 0 ... -4 %.
 constexpr int kNumCus = 256;  // MI355X
-inline int slice_chunk_for(int slices, int groups_per_slice, int resident)
+inline int slice_chunk_for(int slices, int groups_per_slice, int resident, int step = 8)
 {
     if (slices <= 0 || groups_per_slice <= 0) return 1;
     const long long want = (2LL * resident + groups_per_slice - 1) / groups_per_slice;
-    for (long long c = (want + 7) / 8 * 8; c < slices; c += 8)
+    for (long long c = (want + step - 1) / step * step; c < slices; c += step)
         if (slices % c == 0) return (int)c;
     return slices;
+}
+
+// slice_chunk and group_xcd of a launch: with grouped K/V heads the chunks are multiples of 8 G slices where the slice
+// count allows, so that the heads of a K/V head can share an XCD (slice_of_position)
+inline void set_slice_order(FwdArgs& b, int groups_per_slice, int resident)
+{
+    const int slices = b.B * b.H;
+    b.group_xcd = 0;
+    if (b.kv_group > 1 && slices % (8 * b.kv_group) == 0) {
+        b.slice_chunk = slice_chunk_for(slices, groups_per_slice, resident, 8 * b.kv_group);
+        if (b.slice_chunk % (8 * b.kv_group) == 0) b.group_xcd = b.kv_group;
+    } else {
+        b.slice_chunk = slice_chunk_for(slices, groups_per_slice, resident);
+    }
 }
 
 template <int D, int NB, int VAR>
@@ -811,7 +825,7 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
     const long long groups = (long long)a.Tr * a.B * a.H * a.num_splits;
     FwdArgs b = a;
     constexpr int kResident = (NB == 1 && D <= 64 && (VAR & kVarVec) != 0 ? 3 : 2) * kNumCus;
-    b.slice_chunk = slice_chunk_for(a.B * a.H, a.Tr * a.num_splits, kResident);
+    set_slice_order(b, a.Tr * a.num_splits, kResident);
     b.snake_end = snake_end_for(groups, kResident);
     return launch_kernel(kern, dim3((unsigned)groups), dim3(256), smem, st, b);
 }

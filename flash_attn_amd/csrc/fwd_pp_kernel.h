@@ -93,7 +93,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         const int per_chunk = a.slice_chunk * a.Tr * a.num_splits;
         const int pos = work_position(blockIdx.x, a.snake_end);  // (one work-group per CU: the identity)
         const int ch = pos / per_chunk, w = pos % per_chunk;
-        bh = ch * a.slice_chunk + w % a.slice_chunk;
+        bh = ch * a.slice_chunk + slice_of_position(w % a.slice_chunk, a.group_xcd);
         rest = w / a.slice_chunk;
     }
     const int split = rest % a.num_splits;
@@ -644,7 +644,7 @@ inline hipError_t launch_fwd_pp_instance(const FwdArgs& a, hipStream_t st)
     FwdArgs b = a;
     b.Tr = (a.Nq + C::BR - 1) / C::BR;
     const long long groups = (long long)b.Tr * a.B * a.H * a.num_splits;
-    b.slice_chunk = slice_chunk_for(a.B * a.H, b.Tr * a.num_splits, kNumCus);  // one work-group per CU at a time
+    set_slice_order(b, b.Tr * a.num_splits, kNumCus);  // one work-group per CU at a time
     b.snake_end = snake_end_for(groups, kNumCus);
     return launch_kernel(kern, dim3((unsigned)groups), dim3(512), C::SMEM, st, b);
 }

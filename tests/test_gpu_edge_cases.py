@@ -258,14 +258,22 @@ def test_splitkv_heuristic_and_decode_variants(fa, oracle):
     (6, 3, 200, 333, 64, dict()),                    # 4-wave kernel, Nq != Nk
     (4, 1, 129, 129, 31, dict(window=(40, 10))),     # multi-query, element-wise head dim
     (8, 4, 64, 500, 96, dict(causal=True)),
+    # slice counts that are multiples of 8 x (query heads per K/V head): the slice order keeps the heads of a K/V head
+    # on one XCD (a permutation of the slices inside a chunk, in both tiled kernels and in split mode)
+    (16, 4, 300, 300, 128, dict(causal=True)),
+    (64, 8, 140, 200, 64, dict()),
+    (32, 16, 333, 333, 128, dict(causal=True, kernel_hint=2)),
+    (48, 2, 70, 130, 32, dict(window=(50, 20))),
 ])
 def test_grouped_query_heads(fa, oracle, H, Hk, Nq, Nk, d, kw):
     B = 2
+    hint = dict(kernel_hint=kw.pop("kernel_hint")) if "kernel_hint" in kw else {}
     q = randn_f16_gpu((B, H, Nq, d), 11)
     k = randn_f16_gpu((B, Hk, Nk, d), 12)
     v = randn_f16_gpu((B, Hk, Nk, d), 13)
     kr, vr = (t.repeat_interleave(H // Hk, dim=1).contiguous() for t in (k, v))
     O, L = oracle_forward_batched(oracle, q, kr, vr, **kw)
+    kw.update(hint)
     o, lse = fa.flash_forward(q, k, v, **kw)
     check_o_lse(o, lse, O, L, f"GQA H={H} Hk={Hk} tiled")
     # the same through split-KV (tiled split kernel + combine)
