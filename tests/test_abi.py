@@ -167,6 +167,32 @@ def test_split_resolution_and_workspace(fa):
         fa.resolve_splits(1, 1, 1, 128, 64, 1000)
 
 
+def test_automatic_split_count_stays_in_range_on_random_shapes(fa):
+    """2000 random shapes and masks through the host-side resolution (no GPU): the count is at least 1, at most
+    FLASH_MAX_SPLITS and at most the number of 128-key blocks, an explicit count is honoured up to those limits, and the
+    workspace sizes are those of the count.  (tests/test_sanitizers.py runs this file against the instrumented build.)"""
+    rng = np.random.default_rng(5)
+    for it in range(2000):
+        d = int(rng.choice([8, 31, 32, 40, 64, 72, 96, 100, 128]))
+        B, H = int(rng.integers(1, 9)), int(rng.choice([1, 2, 3, 8, 16, 40, 64]))
+        Nq = int(rng.choice([1, 2, 16, 100, 128, 129, 512, 1000, 4096, 20000]))
+        Nk = int(rng.choice([1, 64, 127, 128, 129, 1000, 4096, 30000, 131072, 1 << 20]))
+        if 2 * Nk * d >= 1 << 32 or 2 * Nq * d >= 1 << 32:
+            continue
+        causal = bool(rng.integers(0, 2))
+        window = (int(rng.choice([-1, 0, 5, 256, 5000, 2 ** 31 - 1])), int(rng.choice([-1, 0, 7, 1024, 2 ** 31 - 1])))
+        Hk = int(rng.choice([h for h in (1, 2, 4, 8, H) if H % h == 0]))
+        n_blocks = (Nk + 127) // 128
+        s = fa.resolve_splits(B, H, Nq, Nk, d, 0, causal=causal, window=window, H_kv=Hk)
+        assert 1 <= s <= min(fa.FLASH_MAX_SPLITS, max(1, n_blocks)), (B, H, Nq, Nk, d, causal, window, Hk, s)
+        want = int(rng.integers(1, fa.FLASH_MAX_SPLITS + 1))
+        got = fa.resolve_splits(B, H, Nq, Nk, d, want, causal=causal, window=window, H_kv=Hk)
+        assert got == min(want, max(1, n_blocks))
+        ob, lb = fa.workspace_bytes(B, H, Nq, Nk, d, want, causal=causal, window=window, H_kv=Hk)
+        rows = B * H * got * Nq if got > 1 else 0
+        assert (ob, lb) == (rows * d * 4, rows * 4)
+
+
 def test_stage_stamp_buffer_size(fa):
     L = fa.lib()
     nb = C.c_size_t(99)
