@@ -269,7 +269,7 @@ def stage_stamp_names():
             "tiles<<32|xcc<<16|hw_id", "shader_cycles_first_barrier_to_loop_done")
 
 
-def _shape_params(B, H, Nq, Nk, d, num_splits, causal=False, window=(-1, -1), H_kv=0):
+def _shape_params(B, H, Nq, Nk, d, num_splits, causal=False, window=(-1, -1), H_kv=0, kernel_hint=KERNEL_AUTO):
     p = FlashParams()
     lib().flash_params_init(C.byref(p))
     p.B, p.H, p.Nq, p.Nk, p.d = B, H, Nq, Nk, d
@@ -278,20 +278,23 @@ def _shape_params(B, H, Nq, Nk, d, num_splits, causal=False, window=(-1, -1), H_
     p.is_causal = int(bool(causal))
     p.window_left, p.window_right = int(window[0]), int(window[1])
     p.H_kv = int(H_kv)
+    p.kernel_hint = int(kernel_hint)
     return p
 
 
-def resolve_splits(B, H, Nq, Nk, d, num_splits=0, causal=False, window=(-1, -1), H_kv=0):
+def resolve_splits(B, H, Nq, Nk, d, num_splits=0, causal=False, window=(-1, -1), H_kv=0, kernel_hint=KERNEL_AUTO):
     """The split count flash_forward_splitkv will use for such a call (num_splits <= 0: the library's choice)."""
-    rc = lib().flash_splitkv_resolve_splits(C.byref(_shape_params(B, H, Nq, Nk, d, num_splits, causal, window, H_kv)))
+    rc = lib().flash_splitkv_resolve_splits(C.byref(_shape_params(B, H, Nq, Nk, d, num_splits, causal, window, H_kv,
+                                                                kernel_hint)))
     if rc < 0:
         raise FlashError(rc, "flash_splitkv_resolve_splits")
     return rc
 
 
-def workspace_bytes(B, H, Nq, Nk, d, num_splits=0, causal=False, window=(-1, -1), H_kv=0):
+def workspace_bytes(B, H, Nq, Nk, d, num_splits=0, causal=False, window=(-1, -1), H_kv=0, kernel_hint=KERNEL_AUTO):
     ob, lb = C.c_size_t(), C.c_size_t()
-    rc = lib().flash_splitkv_workspace_bytes(C.byref(_shape_params(B, H, Nq, Nk, d, num_splits, causal, window, H_kv)),
+    rc = lib().flash_splitkv_workspace_bytes(C.byref(_shape_params(B, H, Nq, Nk, d, num_splits, causal, window, H_kv,
+                                                                kernel_hint)),
                                              C.byref(ob), C.byref(lb))
     if rc != FLASH_OK:
         raise FlashError(rc, "flash_splitkv_workspace_bytes")
