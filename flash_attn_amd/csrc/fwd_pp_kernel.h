@@ -184,8 +184,10 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     {
         const int slot = lane & 15;
         const int sigma = 2 * (dkey & 3) + ((dkey >> 2) & 1);
-        kgo = (uint32_t)((tile_begin * BC + dkey) * d * 2 + ((slot ^ (dkey & 15)) << 4));
-        vgo = (uint32_t)((tile_begin * BC + dkey) * d * 2 + ((((slot >> 1) ^ sigma) << 5) | ((slot & 1) << 4)));
+        // (unsigned: a slice may be just short of 4 GiB)
+        const uint32_t row0 = (uint32_t)(tile_begin * BC + dkey) * (uint32_t)(d * 2);
+        kgo = row0 + (uint32_t)((slot ^ (dkey & 15)) << 4);
+        vgo = row0 + (uint32_t)((((slot >> 1) ^ sigma) << 5) | ((slot & 1) << 4));
     }
     const char* const Kb = reinterpret_cast<const char*>(Kbh);
     const char* const Vb = reinterpret_cast<const char*>(Vbh);
@@ -507,7 +509,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         for (int x = 0; x < 8; ++x) {
             const int rl = 4 * x + (lane >> 4);  // row of the wave's 32
             const int gi = q0 + rblk * 32 + rl;
-            const uint32_t off = (uint32_t)((gi < Nq ? gi : Nq - 1) * d * 2 + (((lane & 15) ^ (rl & 15)) << 4));
+            const uint32_t off = (uint32_t)(gi < Nq ? gi : Nq - 1) * (uint32_t)(d * 2) + (uint32_t)(((lane & 15) ^ (rl & 15)) << 4);
             dma_kib(Qb, off, qst + x * 1024);
         }
         if (ntiles > 0) {

@@ -454,6 +454,80 @@ def test_full_size_properties_decode(fa):
     assert torch.allclose(o.float(), torch.full_like(o, 0.5, dtype=torch.float32), atol=1e-3)
 
 
+def _torch_reference_long_keys(q, k, v, lo, hi):
+    """softmax(q k^T / sqrt(d)) v over the keys lo[i] <= j <= hi[i] of one head slice, fp32 on the GPU, keys in chunks
+    (running maximum / sum), for shapes far too long for the CPU oracle.  q [Nq,d], k, v [Nk,d]; returns (O, LSE)."""
+    import torch
+    Nq, d = q.shape
+    Nk = k.shape[0]
+    qf = q.float() * d ** -0.5
+    m = torch.full((Nq,), float("-inf"), device=q.device, dtype=torch.float64)
+    l = torch.zeros((Nq,), device=q.device, dtype=torch.float64)
+    o = torch.zeros((Nq, d), device=q.device, dtype=torch.float64)
+    step = 1 << 20
+    for j0 in range(0, Nk, step):
+        j1 = min(Nk, j0 + step)
+        if int(hi.max()) < j0 or int(lo.min()) >= j1:
+            continue
+        sc = (qf @ k[j0:j1].float().T).double()
+        j = torch.arange(j0, j1, device=q.device)
+        sc = sc.masked_fill((j[None, :] < lo[:, None]) | (j[None, :] > hi[:, None]), float("-inf"))
+        m_new = torch.maximum(m, sc.max(1).values)
+        safe = torch.where(torch.isinf(m_new), torch.zeros_like(m_new), m_new)
+        p = torch.exp(sc - safe[:, None])
+        alpha = torch.where(torch.isinf(m), torch.zeros_like(m), torch.exp(m - safe))
+        l = l * alpha + p.sum(1)
+        o = o * alpha[:, None] + p @ v[j0:j1].double()
+        m = m_new
+    return (o / l[:, None]).float(), (m + torch.log(l)).float()
+
+
+def test_largest_key_count(fa):
+    """The longest K / V the C ABI accepts at d = 128 (a head slice just short of 4 GiB: the kernels address it with
+    32-bit byte offsets), two head slices, so that the second one lies beyond 4 GiB from the tensor's start.  Keys at the
+    start, around the 2 GiB mark and at the very end share a direction with every query (scores around 17 against 0 +- 0.7
+    elsewhere) and carry nearly all of the softmax mass in three equal parts, so that a wrong address there moves O and LSE.
+    Checked against an fp32/fp64 torch evaluation on the GPU (inputs from torch's generator: at this size neither the
+    portable generator nor the CPU oracle finishes in test time): decode, both tiled kernels in split mode, and a
+    causal sliding window at the far end, whose work-groups start at the last tiles."""
+    import torch
+    d, H = 128, 2
+    Nk = (1 << 24) - 128
+    assert 2 * Nk * d < 1 << 32 <= 2 * (Nk + 128) * d
+    g = torch.Generator(device="cuda").manual_seed(5)
+    k = torch.randn((1, H, Nk, d), generator=g, device="cuda", dtype=torch.float16) * 0.5
+    v = torch.randn((1, H, Nk, d), generator=g, device="cuda", dtype=torch.float16)
+    u = torch.where(torch.rand(d, generator=g, device="cuda") < 0.5, -1.0, 1.0).half()  # |u|^2 = d
+    for a, b in ((0, 256), ((1 << 23) - 128, (1 << 23) + 128), (Nk - 256, Nk)):
+        k[:, :, a:b] += 1.5 * u
+    with pytest.raises(fa.FlashError):  # one 128-key block more is refused
+        fa.resolve_splits(1, H, 1, Nk + 128, d)
+
+    def check(o, lse, q, lo, hi, what):
+        for h in range(H):
+            o_ref, l_ref = _torch_reference_long_keys(q[0, h], k[0, h], v[0, h], lo, hi)
+            check_o_lse(o[0, h], lse[0, h], to_f32_np(o_ref), to_f32_np(l_ref), f"{what} head {h}")
+
+    # decode
+    q1 = torch.randn((1, H, 1, d), generator=g, device="cuda", dtype=torch.float16) + u
+    full = (torch.zeros(1, device="cuda", dtype=torch.long), torch.full((1,), Nk - 1, device="cuda", dtype=torch.long))
+    o, lse = fa.flash_forward_splitkv(q1, k, v, num_splits=0)
+    check(o, lse, q1, *full, "decode")
+    # tiled kernels, split over the keys
+    Nq = 300
+    q = torch.randn((1, H, Nq, d), generator=g, device="cuda", dtype=torch.float16) + u
+    lo = torch.zeros(Nq, device="cuda", dtype=torch.long)
+    hi = torch.full((Nq,), Nk - 1, device="cuda", dtype=torch.long)
+    for hint in (fa.KERNEL_4WAVE, fa.KERNEL_8WAVE):
+        o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=64, kernel_hint=hint)
+        check(o, lse, q, lo, hi, f"split, kernel hint {hint}")
+    # causal + left window at the far end (rows are aligned to the end of the keys), unsplit
+    i = torch.arange(Nq, device="cuda") + (Nk - Nq)
+    for hint in (fa.KERNEL_4WAVE, fa.KERNEL_8WAVE):
+        o, lse = fa.flash_forward(q, k, v, causal=True, window=(1000, -1), kernel_hint=hint)
+        check(o, lse, q, i - 1000, i, f"window at the end, kernel hint {hint}")
+
+
 # The 8-wave kernel (d = 128; by preference only large grids of long rows, forced here through kernel_hint):
 # ragged lengths, Nq != Nk in both directions, every mask incl. narrow windows, grouped heads, dropout, split mode.
 @pytest.mark.parametrize("Nq,Nk,Hk,kw", [
