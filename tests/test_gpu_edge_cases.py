@@ -528,6 +528,46 @@ def test_largest_key_count(fa):
         check(o, lse, q, i - 1000, i, f"window at the end, kernel hint {hint}")
 
 
+def test_largest_query_count(fa):
+    """The longest Q / O the C ABI accepts at d = 128 (2^24 - 128 rows: a head slice just short of 4 GiB) over 200 keys,
+    two head slices, both tiled kernels, plain and causal (rows are aligned to the end of the keys: all but the last 200
+    rows see no key and must come back as O = 0, LSE = -inf), against torch fp32 on the GPU."""
+    import torch
+    d, H, Nk = 128, 2, 200
+    Nq = (1 << 24) - 128
+    g = torch.Generator(device="cuda").manual_seed(6)
+    q = torch.randn((1, H, Nq, d), generator=g, device="cuda", dtype=torch.float16)
+    k = torch.randn((1, H, Nk, d), generator=g, device="cuda", dtype=torch.float16)
+    v = torch.randn((1, H, Nk, d), generator=g, device="cuda", dtype=torch.float16)
+    with pytest.raises(fa.FlashError):
+        fa.resolve_splits(1, H, Nq + 128, Nk, d)
+    tail = 4096  # rows compared in full: the first and the last `tail` of every slice (the last ones lie beyond 4 GiB - 1 MiB)
+    for hint in (fa.KERNEL_4WAVE, fa.KERNEL_8WAVE):
+        o, lse = fa.flash_forward(q, k, v, kernel_hint=hint)
+        oc, lsec = fa.flash_forward(q, k, v, causal=True, kernel_hint=hint)
+        for h in range(H):
+            for rows in (slice(0, tail), slice(Nq - tail, Nq)):
+                sc = (q[0, h, rows].float() @ k[0, h].float().T) * d ** -0.5
+                o_ref = torch.softmax(sc, -1) @ v[0, h].float()
+                check_o_lse(o[0, h, rows], lse[0, h, rows], to_f32_np(o_ref), to_f32_np(torch.logsumexp(sc, -1)),
+                            f"hint {hint} head {h} rows {rows}")
+            # every row at once, cheaply: the row sums of O and the LSE against fp32 torch in chunks
+            for r0 in range(0, Nq, 1 << 21):
+                r1 = min(Nq, r0 + (1 << 21))
+                sc = (q[0, h, r0:r1].float() @ k[0, h].float().T) * d ** -0.5
+                assert torch.allclose(lse[0, h, r0:r1], torch.logsumexp(sc, -1), atol=1e-4)
+                osum = (torch.softmax(sc, -1) @ v[0, h].float().sum(-1, keepdim=True))[:, 0]
+                assert torch.allclose(o[0, h, r0:r1].float().sum(-1), osum, atol=2e-2)
+            # causal: rows before Nq - Nk see nothing
+            assert torch.isneginf(lsec[0, h, :Nq - Nk]).all() and not o[0, h, :0].any()
+            assert not oc[0, h, :Nq - Nk].any()
+            i = torch.arange(Nq - Nk, Nq, device="cuda")
+            sc = (q[0, h, Nq - Nk:].float() @ k[0, h].float().T) * d ** -0.5
+            sc = sc.masked_fill(torch.arange(Nk, device="cuda")[None, :] > (i - (Nq - Nk))[:, None], float("-inf"))
+            check_o_lse(oc[0, h, Nq - Nk:], lsec[0, h, Nq - Nk:], to_f32_np(torch.softmax(sc, -1) @ v[0, h].float()),
+                        to_f32_np(torch.logsumexp(sc, -1)), f"causal hint {hint} head {h}")
+
+
 # The 8-wave kernel (d = 128; by preference only large grids of long rows, forced here through kernel_hint):
 # ragged lengths, Nq != Nk in both directions, every mask incl. narrow windows, grouped heads, dropout, split mode.
 @pytest.mark.parametrize("Nq,Nk,Hk,kw", [
