@@ -54,6 +54,7 @@ struct FwdArgs {
     int slice_chunk;     // head slices per chunk of the work-group order (set by the kernel's launcher)
     int snake_end;       // work-groups below this index sit on the GPU together; odd 256-blocks of them run reversed (launcher)
     int group_xcd;       // > 1: query heads per K/V head, and the slice order keeps the heads of a K/V head on one XCD (launcher)
+    int split_rotate;    // 1: the split index of a work-group is rotated by its row block (launcher; split_of_rest)
 
     // index of the K/V slice [Nk,d] read by query slice bh = b * H + h
     __device__ __forceinline__ int kv_slice(int bh) const { return (bh / H) * Hk + (bh % H) / kv_group; }
@@ -86,6 +87,25 @@ __device__ __forceinline__ int work_position(int block, int snake_end)
 // 3.7 times the K/V/Q bytes fetched).  Instead position (x, y) = (p % 8, p / 8) takes query head y % G of K/V slice
 // 8 (y / G) + x: the heads of a K/V head share an XCD and follow each other there.  A bijection on chunks whose size is
 // a multiple of 8 G (the launcher sets group_xcd only then).
+// Split index and row-block index of the position `rest` inside a slice (splits fastest).  Where the slices of a chunk
+// are not a multiple of 8, the XCD of a work-group depends on its split: with 4 slices and 2 splits, XCDs 0-3 get
+// every first split and XCDs 4-7 every second one, and under a causal mask, whose first splits are the long ones, half the
+// chip then carries three quarters of the work (measured B1 H4 N16384 d32 causal, 2 splits: 201 us, against 160 us
+// unsplit and 158 us with 5 splits).  Rotating the split index by the row-block index deals every split to every XCD.
+// The launcher asks for it exactly where the plain order aliases: work-group x + 8 n of XCD x has split
+// (x / c + (8 / c) n) % S for c = 1, 2 or 4 slices per chunk, which reaches every split only if S is odd; other chunk
+// sizes mix by themselves, and rotating an order that already mixes measured 0 ... -14 %.
+__device__ __forceinline__ int split_of_rest(int rest, int num_splits, int rotate, int* row_block_index)
+{
+    const int mi = rest / num_splits, s0 = rest % num_splits;
+    *row_block_index = mi;
+    return rotate ? (s0 + mi) % num_splits : s0;
+}
+inline int split_rotate_for(int num_splits, int slice_chunk)
+{
+    return num_splits > 1 && num_splits % 2 == 0 && (slice_chunk == 1 || slice_chunk == 2 || slice_chunk == 4) ? 1 : 0;
+}
+
 __device__ __forceinline__ int slice_of_position(int local, int group_xcd)
 {
     if (group_xcd > 1) {

@@ -132,8 +132,9 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
         bh = ch * a.slice_chunk + slice_of_position(w % a.slice_chunk, a.group_xcd);
         rest = w / a.slice_chunk;
     }
-    const int split = rest % a.num_splits;
-    const int m_block = a.Tr - 1 - rest / a.num_splits;
+    int mi;
+    const int split = split_of_rest(rest, a.num_splits, a.split_rotate, &mi);
+    const int m_block = a.Tr - 1 - mi;
     const int h = bh % a.H;
     const int Nq = a.Nq, Nk = a.Nk, d = kFullD ? D : a.d;
     const int shift = Nk - Nq;
@@ -826,6 +827,7 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
     FwdArgs b = a;
     constexpr int kResident = (NB == 1 && D <= 64 && (VAR & kVarVec) != 0 ? 3 : 2) * kNumCus;
     set_slice_order(b, a.Tr * a.num_splits, kResident);
+    b.split_rotate = split_rotate_for(b.num_splits, b.slice_chunk);
     b.snake_end = snake_end_for(groups, kResident);
     return launch_kernel(kern, dim3((unsigned)groups), dim3(256), smem, st, b);
 }

@@ -96,8 +96,9 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         bh = ch * a.slice_chunk + slice_of_position(w % a.slice_chunk, a.group_xcd);
         rest = w / a.slice_chunk;
     }
-    const int split = rest % a.num_splits;
-    const int m_block = a.Tr - 1 - rest / a.num_splits;
+    int mi;
+    const int split = split_of_rest(rest, a.num_splits, a.split_rotate, &mi);
+    const int m_block = a.Tr - 1 - mi;
     const int h = bh % a.H;
     const int Nq = a.Nq, Nk = a.Nk;
     constexpr int d = D;
@@ -647,6 +648,7 @@ inline hipError_t launch_fwd_pp_instance(const FwdArgs& a, hipStream_t st)
     b.Tr = (a.Nq + C::BR - 1) / C::BR;
     const long long groups = (long long)b.Tr * a.B * a.H * a.num_splits;
     set_slice_order(b, b.Tr * a.num_splits, kNumCus);  // one work-group per CU at a time
+    b.split_rotate = split_rotate_for(b.num_splits, b.slice_chunk);
     b.snake_end = snake_end_for(groups, kNumCus);
     return launch_kernel(kern, dim3((unsigned)groups), dim3(512), C::SMEM, st, b);
 }

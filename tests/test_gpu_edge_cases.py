@@ -185,6 +185,25 @@ def test_general_splitkv_matches_unsplit(fa, oracle, S):
             assert np.abs(op - Ot).max() <= 2e-3
 
 
+@pytest.mark.parametrize("H", [1, 2, 4, 8, 3])
+@pytest.mark.parametrize("S", [2, 4, 6])
+def test_split_index_rotation(fa, oracle, H, S):
+    """1, 2 or 4 head slices with an even split count: the kernels deal the splits to the XCDs by rotating the split
+    index with the row block.  Every partial must still be the one the oracle computes for that split index (same
+    layout [B,H,S,Nq,d]); 8 and 3 slices take the plain order."""
+    B, N, d = 1, 777, 64
+    q, k, v = _qkv(B, H, N, N, d, seed=40 + H + S)
+    o, lse, ws = fa.flash_forward_splitkv(q, k, v, num_splits=S, causal=True, return_partials=True)
+    O, L = oracle_forward_batched(oracle, q, k, v, causal=True)
+    check_o_lse(o, lse, O, L, f"H={H} S={S}")
+    Ot, Ls, Ms, LSEp = oracle.splitkv_partials(to_f32_np(q), to_f32_np(k), to_f32_np(v), S, causal=True)
+    op, lp = to_f32_np(ws[0]), to_f32_np(ws[1])
+    assert np.array_equal(np.isneginf(lp), np.isneginf(LSEp))
+    fin = np.isfinite(LSEp)
+    assert np.abs(lp[fin] - LSEp[fin]).max() <= 1e-4
+    assert np.abs(op - Ot).max() <= 2e-3
+
+
 @pytest.mark.parametrize("B,H,Nq,Nk,d,causal,want", [
     (1, 8, 512, 32768, 128, False, 16),   # long keys, small batch: two work-groups per CU
     (1, 32, 128, 16384, 128, True, 8),    # causal with Nq < Nk: every split holds visible keys
@@ -607,8 +626,9 @@ def test_eight_wave_kernel_cases(fa, oracle, Nq, Nk, Hk, kw):
     O, L = oracle_forward_batched(oracle, q, kr, vr, **okw)
     check_o_lse(o, lse, O, L, f"8-wave Nq={Nq} Nk={Nk} {sorted(kw)}")
     if p == 0.0:
-        o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=3, **kw)
-        check_o_lse(o, lse, O, L, f"8-wave split Nq={Nq} Nk={Nk} {sorted(kw)}")
+        for S in (3, 4):  # (an even count over two slices: the split index is rotated by the row block)
+            o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=S, **kw)
+            check_o_lse(o, lse, O, L, f"8-wave split S={S} Nq={Nq} Nk={Nk} {sorted(kw)}")
 
 
 @pytest.mark.parametrize("Nq,Nk,d,Hk,kw", [
