@@ -479,6 +479,15 @@ def main():
                 fl = flops_of(c2)
                 others[n2] = {"workload": DESCR[n2], "ms": ev, "TFLOP/s": fl / (ev * 1e-3) / 1e12,
                               "frac_mfma_peak": fl / (ev * 1e-3) / 1e12 / PEAK_F16_TFLOPS, "algorithmic_flops": fl}
+            if n2 == "cfg5":
+                # the same launch with the library's own split count (num_splits = 0) instead of the 16 the configuration names
+                c3 = dict(c2, splits=-1)
+                st3, _ = make_step(fa, c3, q, k, v)
+                _, ev3 = time_steps(st3, steps2, 10)
+                others[n2]["automatic_split_count"] = {
+                    "splits": fa.resolve_splits(c2["B"], c2["H"], c2["Nq"], c2["Nk"], c2["d"], 0), "ms": ev3,
+                    "GB/s": by / (ev3 * 1e-3) / 1e9, "frac_hbm_peak": by / (ev3 * 1e-3) / 1e9 / PEAK_HBM_GBPS}
+                del st3
             if not args.no_cpu:
                 others[n2]["cpu_baseline"] = cpu_baseline(c2, q, k, v, args.cpu_slices or CPU_SLICES[n2])
             del q, k, v, st
@@ -487,7 +496,8 @@ def main():
             result["roofline_decode"] = {"bound": "hbm", "achieved": others["cfg5"]["GB/s"], "peak": PEAK_HBM_GBPS,
                                          "unit": "GB/s", "frac": others["cfg5"]["frac_hbm_peak"],
                                          "traffic": measured_traffic("cfg5"),
-                                         "traffic_source": f"profiles/{PROFILE_OF['cfg5']}"}
+                                         "traffic_source": f"profiles/{PROFILE_OF['cfg5']}",
+                                         "automatic_split_count": others["cfg5"]["automatic_split_count"]}
             if "cpu_baseline" in others["cfg5"]:
                 result["roofline_decode"]["cpu_baseline"] = others["cfg5"]["cpu_baseline"]
     print(json.dumps(result))

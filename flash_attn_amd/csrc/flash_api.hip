@@ -263,19 +263,48 @@ int resolve_splits(const flash_params* p)
     const int n_blocks = (p->Nk + FLASH_SPLIT_KEY_GRANULE - 1) / FLASH_SPLIT_KEY_GRANULE;
     int s = p->num_splits;
     if (s <= 0 && p->Nq == 1) {
-        // Decode streams K and V once and is bound by HBM: the reference's rule (fill the SMs once) leaves most of the
-        // bandwidth unused here, where one 256-thread work-group keeps far fewer bytes in flight than a CU can.
-        // Measured on 256 CUs, as long as a split still streams 512 keys or more: the one-row kernel keeps gaining up
-        // to about 32 work-groups per CU in the launch; the tiled kernel, which takes over when four or more query
-        // heads of a K/V head decode together (flash_forward_splitkv: one work-group per K/V head and split), is best
-        // near 2 per CU and loses 10-30 % beyond 8.
+        // Decode.  The reference's rule (fill the SMs once) leaves most of the bandwidth unused here: a lone work-group
+        // of the one-row kernel streams 13-16 GB/s, far fewer bytes in flight than a CU can keep.
         const int hk = p->H_kv > 0 ? p->H_kv : p->H;
-        const bool grouped = p->H / (hk > 0 ? hk : 1) >= 4;
-        const long long base = (long long)p->B * (grouped ? hk : p->H);
-        const long long target = (grouped ? 2LL : 32LL) * kNumCU;
-        const long long want = (target + base - 1) / (base > 0 ? base : 1);
-        const int by_keys = n_blocks / 4;  // 512 keys per split
-        s = (int)(want < by_keys ? want : by_keys);
+        const int G = p->H / (hk > 0 ? hk : 1);
+        const bool heads_as_rows = G >= 4 && !p->alibi_slopes && window_left_of(p) < 0 && p->dropout_p == 0.0f;
+        const bool one_row_kernel = !heads_as_rows && p->d % 8 == 0 && p->dropout_p == 0.0f && p->softmax_scale > 0.0f;
+        if (one_row_kernel) {
+            // Measured over 120 random shapes and 17 large ones on 256 CUs: the launch is fastest with about four query
+            // heads x splits per CU whatever the batch, heads and key count (B16 H32 Nk16384 d128: 1 / 2 / 3 / 8 / 16 /
+            // 64 splits 787 / 609 / 614 / 637 / 634 / 686 us; B1 H32: best at 32), 10-20 % slower at exactly eight per CU
+            // (B16 H32, 4 splits: 699 us; B64 H32 unsplit 697 against 631 with 3 or 4); and every split adds to the
+            // combine, which bounds the useful count by about sqrt(Nk / 3) (B2 H1 Nk16384: 64 splits 17.5 us, 128: 25.6).
+            // A head dim below the width of its instance (128 / 64 / 32 lanes' worth per key) leaves lanes idle and fewer bytes
+            // in flight per work-group: the target grows by width / d (d = 96 and 72, 128 heads: 12 splits 8-15 % faster than 8).
+            const long long heads = (long long)p->B * p->H;
+            const int width = p->d > 64 ? 128 : p->d > 32 ? 64 : 32;
+            const long long target = 4LL * kNumCU * width / p->d;
+            long long want = (2 * target + heads) / (2 * (heads > 0 ? heads : 1));  // round(target / heads)
+            if (want < 1) want = 1;
+            if (want == 1 && heads > 7 * kNumCU && heads < 8 * kNumCU + kNumCU / 2) want = 3;
+            long long cap = FLASH_MAX_SPLITS;
+            while (cap > 1 && cap * cap * 3 > (long long)p->Nk) --cap;  // cap <= sqrt(Nk / 3)
+            if (want > cap) want = cap;
+            s = (int)(want < n_blocks ? want : n_blocks);
+        } else {
+            // The tiled kernel serves four or more query heads of a K/V head together (heads as the rows of one problem per
+            // K/V head) and every request the one-row kernel cannot (d % 8 != 0, dropout): the estimate of the tiled path
+            // for that problem.
+            flash_params r = *p;
+            if (heads_as_rows) {
+                r.H = hk;
+                r.H_kv = 0;
+                r.Nq = G;
+                r.is_causal = 0;
+                r.window_right = -1;
+            }
+            s = auto_splits_tiled(&r, n_blocks);
+        }
+        if (s >= 1) {  // the count whose splits are all non-empty (src/main.cu:397-398 skips the others too)
+            const int per = (n_blocks + s - 1) / s;
+            s = (n_blocks + per - 1) / per;
+        }
     } else if (s <= 0) {
         s = auto_splits_tiled(p, n_blocks);
     }
