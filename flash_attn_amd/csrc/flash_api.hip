@@ -270,21 +270,18 @@ int resolve_splits(const flash_params* p)
         const bool heads_as_rows = G >= 4 && !p->alibi_slopes && window_left_of(p) < 0 && p->dropout_p == 0.0f;
         const bool one_row_kernel = !heads_as_rows && p->d % 8 == 0 && p->dropout_p == 0.0f && p->softmax_scale > 0.0f;
         if (one_row_kernel) {
-            // Measured over 120 random shapes and 17 large ones on 256 CUs: the launch is fastest with about four query
-            // heads x splits per CU whatever the batch, heads and key count (B16 H32 Nk16384 d128: 1 / 2 / 3 / 8 / 16 /
-            // 64 splits 787 / 609 / 614 / 637 / 634 / 686 us; B1 H32: best at 32), 10-20 % slower at exactly eight per CU
-            // (B16 H32, 4 splits: 699 us; B64 H32 unsplit 697 against 631 with 3 or 4); and every split adds to the
-            // combine, which bounds the useful count by about sqrt(Nk / 3) (B2 H1 Nk16384: 64 splits 17.5 us, 128: 25.6).
-            // A head dim below the width of its instance (128 / 64 / 32 lanes' worth per key) leaves lanes idle and fewer bytes
-            // in flight per work-group: the target grows by width / d (d = 96 and 72, 128 heads: 12 splits 8-15 % faster than 8).
-            const long long heads = (long long)p->B * p->H;
-            const int width = p->d > 64 ? 128 : p->d > 32 ? 64 : 32;
-            const long long target = 4LL * kNumCU * width / p->d;
-            long long want = (2 * target + heads) / (2 * (heads > 0 ? heads : 1));  // round(target / heads)
+            // Each wave keeps the 2 U loads of its next key block in flight while it works on the current one (64-128 KiB
+            // per work-group), so one work-group per CU already covers the memory latency.  Measured over 61 random
+            // shapes and 10 large ones on 256 CUs: the launch is fastest with about 256 work-groups whatever the batch,
+            // heads and key count (B1 H32 Nk16384 d128: 1 / 4 / 6 / 8 / 16 / 32 splits 142 / 48 / 42 / 42 / 45 / 48 us;
+            // B4 H8 Nk65536: best at 6; B16 H32 and B64 H32: unsplit); and every split adds to the combine, which
+            // bounds the useful count by about sqrt(Nk / 12).
+            const int per_group = G % 8 == 0 ? 8 : G % 4 == 0 ? 4 : G % 2 == 0 ? 2 : 1;  // query heads per work-group
+            const long long groups = (long long)p->B * p->H / per_group;
+            long long want = (2LL * kNumCU + groups) / (2 * (groups > 0 ? groups : 1));  // round(256 / groups)
             if (want < 1) want = 1;
-            if (want == 1 && heads > 7 * kNumCU && heads < 8 * kNumCU + kNumCU / 2) want = 3;
             long long cap = FLASH_MAX_SPLITS;
-            while (cap > 1 && cap * cap * 3 > (long long)p->Nk) --cap;  // cap <= sqrt(Nk / 3)
+            while (cap > 1 && cap * cap * 12 > (long long)p->Nk) --cap;  // cap <= sqrt(Nk / 12)
             if (want > cap) want = cap;
             s = (int)(want < n_blocks ? want : n_blocks);
         } else {
