@@ -278,7 +278,10 @@ int resolve_splits(const flash_params* p)
             // bounds the useful count by about sqrt(Nk / 12).
             const int per_group = G % 8 == 0 ? 8 : G % 4 == 0 ? 4 : G % 2 == 0 ? 2 : 1;  // query heads per work-group
             const long long groups = (long long)p->B * p->H / per_group;
-            long long want = (2LL * kNumCU + groups) / (2 * (groups > 0 ? groups : 1));  // round(256 / groups)
+            // (twice that where a work-group serves four or eight query heads, which only ALiBi or a window send here: it
+            // then spends as long on arithmetic as on loads; B16 H32 H_kv8 Nk16384 with ALiBi 2 / 4 splits 185 / 171 us)
+            const long long target = (per_group >= 4 ? 2LL : 1LL) * kNumCU;
+            long long want = (2 * target + groups) / (2 * (groups > 0 ? groups : 1));  // round(target / groups)
             if (want < 1) want = 1;
             long long cap = FLASH_MAX_SPLITS;
             while (cap > 1 && cap * cap * 12 > (long long)p->Nk) --cap;  // cap <= sqrt(Nk / 12)
