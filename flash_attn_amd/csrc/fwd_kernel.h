@@ -83,6 +83,23 @@ __device__ __forceinline__ v4u load_chunk(const half_t* __restrict__ rowp, int c
     }
 }
 
+// The same for a chunk of a K or V tile, without the zeroes: columns >= d come back as copies of the row's last
+// elements.  For K they meet the zero columns of Q, for V they only reach rows of O^T that are never stored, so the
+// values do not matter as long as they are the row's own finite data -- and without the select the tile's loads are
+// not waited for until their data is written to LDS, behind the arithmetic of the current tile (with it, the compiler
+// placed the selects, and with them the wait for the whole tile, right behind the loads).
+template <bool kVec, bool kFullD>
+__device__ __forceinline__ v4u load_chunk_unpadded(const half_t* __restrict__ rowp, int col, int d)
+{
+    if constexpr (kFullD) {
+        return *reinterpret_cast<const v4u*>(rowp + col);
+    } else if constexpr (kVec) {
+        return *reinterpret_cast<const v4u*>(rowp + (col < d ? col : d - 8));
+    } else {
+        return load_chunk<kVec, kFullD>(rowp, col, d);
+    }
+}
+
 // Running maximum is only raised when some row of the wave outgrows it by more than this many powers of two;
 // until then probabilities are taken relative to the stale maximum (bounded by 2^kLazyTau, exact in the end
 // because numerator and denominator carry the same factor).  Saves the per-tile rescale of the O accumulators.
@@ -206,11 +223,29 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     for (int nb = 0; nb < NB; ++nb) {
         const int ic = row_i[nb] < Nq ? row_i[nb] : Nq - 1;
         const half_t* qrow = Qbh + (size_t)ic * d;
+        if constexpr (kVec) {
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            union { v4u u; v8h h; } t;
-            t.u = load_chunk<kVec, kFullD>(qrow, 16 * ks + 8 * g, d);
-            qf[nb][ks] = t.h;
+            for (int ks = 0; ks < KS; ++ks) {
+                union { v4u u; v8h h; } t;
+                t.u = load_chunk<kVec, kFullD>(qrow, 16 * ks + 8 * g, d);
+                qf[nb][ks] = t.h;
+            }
+        } else {
+            // element-wise rows: every load of the row block first, then the zero padding and the packing (written as
+            // one chunk after the other, each 2-byte load was waited for before the next was issued)
+            half_t raw[KS][8];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int c = 16 * ks + 8 * g + e;
+                    raw[ks][e] = qrow[c < d ? c : d - 1];
+                }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qf[nb][ks][e] = 16 * ks + 8 * g + e < d ? raw[ks][e] : (half_t)0.0f;
         }
     }
 
@@ -222,25 +257,52 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
         ld_row[x] = cid / CH;
         ld_col[x] = (cid % CH) * 8;
     }
-    v4u kreg[NLD], vreg[NLD];
-    auto gload = [&](const half_t* __restrict__ base, int tile, v4u (&reg)[NLD]) {
+    // A staged chunk: the 16 bytes as loaded (rows of 16-byte pieces), or its eight elements one per register (element-wise
+    // rows: packed only where the chunk is written to LDS, behind the arithmetic of the current tile; packed where they
+    // are loaded, the loads of the next tile were waited for before that arithmetic began).  Columns >= d hold copies of
+    // the row's last elements (load_chunk_unpadded).
+    // (Only the 32-wide bucket has the registers for it: at 64 it measured -7 %, at 128, which already spills, -16 %.)
+    constexpr bool kPackLate = !kVec && D <= 32;
+    struct Staged {
+        v4u v;
+        uint32_t e[kPackLate ? 8 : 1];
+    };
+    Staged kreg[NLD], vreg[NLD];
+    auto gload = [&](const half_t* __restrict__ base, int tile, Staged (&reg)[NLD]) {
         const int kb0 = tile * BC;
 #pragma unroll
         for (int x = 0; x < NLD; ++x) {
             const int r = kb0 + ld_row[x];
-            reg[x] = load_chunk<kVec, kFullD>(base + (size_t)(r < Nk ? r : Nk - 1) * d, ld_col[x], d);
+            const half_t* __restrict__ rowp = base + (size_t)(r < Nk ? r : Nk - 1) * d;
+            if constexpr (!kPackLate) {
+                reg[x].v = load_chunk_unpadded<kVec, kFullD>(rowp, ld_col[x], d);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int c = ld_col[x] + e;
+                    reg[x].e[e] = reinterpret_cast<const uint16_t*>(rowp)[c < d ? c : d - 1];
+                }
+            }
+        }
+    };
+    auto staged_chunk = [&](const Staged& r) {
+        if constexpr (!kPackLate) {
+            return r.v;
+        } else {
+            const v4u p = {r.e[0] | (r.e[1] << 16), r.e[2] | (r.e[3] << 16), r.e[4] | (r.e[5] << 16), r.e[6] | (r.e[7] << 16)};
+            return p;
         }
     };
     auto put_k = [&](int buf) {
 #pragma unroll
         for (int x = 0; x < NLD; ++x)
-            *reinterpret_cast<v4u*>(Ks + buf * C::KBUF + ld_row[x] * SK + ld_col[x] * 2) = kreg[x];
+            *reinterpret_cast<v4u*>(Ks + buf * C::KBUF + ld_row[x] * SK + ld_col[x] * 2) = staged_chunk(kreg[x]);
     };
     auto put_v = [&](int buf) {
 #pragma unroll
         for (int x = 0; x < NLD; ++x)
             *reinterpret_cast<v4u*>(Vs + buf * C::VBUF + ld_row[x] * SV +
-                                    ((ld_col[x] * 2) ^ (C::VSWZ ? ((ld_row[x] >> 1) & 1) << 6 : 0))) = vreg[x];
+                                    ((ld_col[x] * 2) ^ (C::VSWZ ? ((ld_row[x] >> 1) & 1) << 6 : 0))) = staged_chunk(vreg[x]);
     };
 
     // ---- direct global -> LDS path: the tile buffers keep their layout (K rows padded by one chunk, V rows with the
