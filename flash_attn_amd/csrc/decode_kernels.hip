@@ -244,7 +244,7 @@ __global__ void __launch_bounds__(256) combine_kernel(const float* __restrict__ 
     const size_t sstride = (size_t)Nq * d;                     // floats between the partial rows of two splits
     const float* op = O_partial + ((size_t)bh * S * Nq + i) * d;
     const bool vec = (d & 7) == 0;  // rows of the partials and of O are 16-byte aligned (the host checks the bases)
-    constexpr int U = 4;            // partial rows in flight per half-wave
+    constexpr int U = 8;            // partial rows in flight per half-wave
     const int c4 = (lane & 31) * 4, grp = lane >> 5;
     const bool act = c4 < d;
     float4 pre[U];
@@ -276,11 +276,21 @@ __global__ void __launch_bounds__(256) combine_kernel(const float* __restrict__ 
             const float w = s < S ? s_w[wave][s] : 0.0f;
             acc.x += w * pre[u].x, acc.y += w * pre[u].y, acc.z += w * pre[u].z, acc.w += w * pre[u].w;
         }
-        if (act) {
-            for (int s = grp + 2 * U; s < S; s += 2) {
-                const float4 o = *reinterpret_cast<const float4*>(op + s * sstride + c4);
-                const float w = s_w[wave][s];
-                acc.x += w * o.x, acc.y += w * o.y, acc.z += w * o.z, acc.w += w * o.w;
+        // the remaining partial rows, U at a time, requested together (one by one, every request waited for its
+        // predecessor's arithmetic: with 64 splits and more the combine took longer than the split kernel)
+        for (int s0 = grp + 2 * U; s0 < S; s0 += 2 * U) {  // (wave-uniform trip count: the first half-wave's)
+            float4 nxt[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int s = s0 + 2 * u;
+                nxt[u] = (act && s < S) ? *reinterpret_cast<const float4*>(op + s * sstride + c4) : float4{0.f, 0.f, 0.f, 0.f};
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int s = s0 + 2 * u;
+                const float w = s < S ? s_w[wave][s] : 0.0f;
+                acc.x += w * nxt[u].x, acc.y += w * nxt[u].y, acc.z += w * nxt[u].z, acc.w += w * nxt[u].w;
             }
         }
         acc.x = xhalf_sum(acc.x), acc.y = xhalf_sum(acc.y), acc.z = xhalf_sum(acc.z), acc.w = xhalf_sum(acc.w);

@@ -185,7 +185,7 @@ long long tiled_groups(const flash_params* p, const fa::FwdArgs& a)
 // 15 %); the reference's rule with 256 CUs: 12 of 21, the worst 6.8 times slower than the best count.  Costs the host
 // up to 0.2 ms on very long sequences (a loop over row blocks per candidate count): callers on a tight loop pass an
 // explicit count, or the one flash_splitkv_resolve_splits returned for the shape.
-int auto_splits_tiled(const flash_params* p, int n_blocks)
+int auto_splits_tiled(const flash_params* p, int n_blocks, bool decode = false)
 {
     const int wl = window_left_of(p), wr = window_right_of(p);
     const bool vec = (tiled_variant(p) & 1) != 0;
@@ -199,13 +199,15 @@ int auto_splits_tiled(const flash_params* p, int n_blocks)
     // (d % 8 == 0 but not the bucket's width), x 3.4 with element-wise loads (d % 8 != 0)
     static const float kTile[5] = {0.0f, 0.5f, 0.72f, 0.88f, 1.0f};
     const bool dma = vec && p->d == 32 * bucket;
-    const float b = pp ? 1.97f : kTile[bucket] * (dma ? 1.0f : vec ? 1.3f : 3.4f);
+    // (decode launches, whose tiles no other work-group has asked for before: twice that, and 0.04 us per split for
+    // the combine of their few rows; fitted to 55 random decode shapes of the tiled routes)
+    const float b = (pp ? 1.97f : kTile[bucket] * (dma ? 1.0f : vec ? 1.3f : 3.4f)) * (decode ? 2.0f : 1.0f);
     const float rho2 = pp ? 1.0f : dma ? 1.32f : vec ? 1.5f : 1.6f;
     const float rho3 = (!pp && vec && p->d <= 64) ? rho2 * 1.12f : rho2;  // three places per CU up to d = 64
     // a: prologue + epilogue of a work-group; c0 + c1 s: the combine launch and what every further split adds to it and to
     // the split launch; partials: 8 B H Nq d bytes written and read back per split at 4.2 TB/s.  (Fitted to sweeps of
     // explicit counts over 101 shapes, checked on 40 others.)
-    const float a = 5.0f, c0 = 4.2f, c1 = 0.09f;
+    const float a = 5.0f, c0 = 4.2f, c1 = decode ? 0.04f : 0.09f;
     const float partials = 8.0f * (float)slices * (float)p->Nq * (float)p->d / 4.2e6f;  // us per split
     const int shift = p->Nk - p->Nq;
     const bool masked = p->is_causal || wl >= 0 || wr >= 0;
@@ -275,7 +277,7 @@ int resolve_splits(const flash_params* p)
             // shapes and 10 large ones on 256 CUs: the launch is fastest with about 256 work-groups whatever the batch,
             // heads and key count (B1 H32 Nk16384 d128: 1 / 4 / 6 / 8 / 16 / 32 splits 142 / 48 / 42 / 42 / 45 / 48 us;
             // B4 H8 Nk65536: best at 6; B16 H32 and B64 H32: unsplit); and every split adds to the combine, which
-            // bounds the useful count by about sqrt(Nk / 12).
+            // bounds the useful count by about sqrt(Nk / 3).
             const int per_group = G % 8 == 0 ? 8 : G % 4 == 0 ? 4 : G % 2 == 0 ? 2 : 1;  // query heads per work-group
             const long long groups = (long long)p->B * p->H / per_group;
             // (twice that where a work-group serves four or eight query heads, which only ALiBi or a window send here: it
@@ -284,7 +286,7 @@ int resolve_splits(const flash_params* p)
             long long want = (2 * target + groups) / (2 * (groups > 0 ? groups : 1));  // round(target / groups)
             if (want < 1) want = 1;
             long long cap = FLASH_MAX_SPLITS;
-            while (cap > 1 && cap * cap * 12 > (long long)p->Nk) --cap;  // cap <= sqrt(Nk / 12)
+            while (cap > 1 && cap * cap * 3 > (long long)p->Nk) --cap;  // cap <= sqrt(Nk / 3)
             if (want > cap) want = cap;
             s = (int)(want < n_blocks ? want : n_blocks);
         } else {
@@ -299,7 +301,7 @@ int resolve_splits(const flash_params* p)
                 r.is_causal = 0;
                 r.window_right = -1;
             }
-            s = auto_splits_tiled(&r, n_blocks);
+            s = auto_splits_tiled(&r, n_blocks, true);
         }
         if (s >= 1) {  // the count whose splits are all non-empty (src/main.cu:397-398 skips the others too)
             const int per = (n_blocks + s - 1) / s;

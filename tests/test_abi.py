@@ -156,7 +156,7 @@ def test_split_resolution_and_workspace(fa):
     assert fa.resolve_splits(1, 2, 16384, 16384, 64, 0, causal=True) == 5
     # a narrow window leaves a row block two or three key blocks: nothing to split
     assert fa.resolve_splits(1, 4, 4096, 4096, 64, 0, window=(256, 0)) == 1
-    # one query row (decode, bandwidth-bound), one-row kernel: about one work-group per CU, at most sqrt(Nk / 12) splits
+    # one query row (decode, bandwidth-bound), one-row kernel: about one work-group per CU, at most sqrt(Nk / 3) splits
     assert fa.resolve_splits(16, 32, 1, 16384, 128, 0) == 1
     assert fa.resolve_splits(1, 32, 1, 16384, 128, 0) == 8
     assert fa.resolve_splits(1, 32, 1, 2048, 128, 0) == 8
@@ -164,7 +164,7 @@ def test_split_resolution_and_workspace(fa):
     assert fa.resolve_splits(1, 8, 1, 1 << 20, 128, 0) == 32
     assert fa.resolve_splits(512, 32, 1, 16384, 128, 0) == 1
     assert fa.resolve_splits(64, 32, 1, 4096, 128, 0) == 1
-    assert fa.resolve_splits(2, 1, 1, 16384, 64, 0) == 32         # few heads: bounded by sqrt(Nk / 12)
+    assert fa.resolve_splits(2, 1, 1, 16384, 64, 0) == 64         # few heads: bounded by sqrt(Nk / 3)
     assert fa.resolve_splits(2, 16, 1, 32768, 128, 0, H_kv=8) == 16   # two query heads per work-group: 16 work-groups per split
     assert fa.resolve_splits(1, 1, 1, 300, 64, 0) == 3
     # grouped heads as the rows of the tiled kernel, and requests the one-row kernel cannot serve: the tiled estimate
