@@ -100,6 +100,33 @@ __device__ __forceinline__ v4u load_chunk_unpadded(const half_t* __restrict__ ro
     }
 }
 
+// Rows that start at any 2-byte boundary (d % 8 != 0), d >= 8: a chunk is still one 16-byte load -- the hardware runs in
+// unaligned access mode -- taken at the chunk's own column, or, for the row's last, partial chunk and for chunks past the
+// row, at column d - 8, so that no load ever leaves the row.  finish_chunk_anyalign turns what was loaded into the chunk
+// at column col: whole chunks as they are; the partial one moved down by 8 - d % 8 elements, which brings zeroes in
+// from the top, exactly its columns >= d; chunks past the row zero.  (Two steps, so that the caller can keep the
+// arithmetic away from the load: see load_chunk_unpadded.)  Element by element, a 64 x 32 tile took 16 two-byte loads
+// per thread with an address computation each, where this takes two loads.
+typedef v4u __attribute__((aligned(2))) v4u_anyalign;
+__device__ __forceinline__ v4u load_chunk_anyalign(const half_t* __restrict__ rowp, int col, int d)
+{
+    return *reinterpret_cast<const v4u_anyalign*>(rowp + (col + 8 <= d ? col : d - 8));
+}
+__device__ __forceinline__ v4u finish_chunk_anyalign(v4u v, int col, int d)
+{
+    const int k = 8 - (d & 7);  // elements to move down by: the same in every lane, 1 ... 7
+    const int ws = k >> 1;      // whole 32-bit words of it
+    uint32_t t[5];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t[i] = ws == 0 ? v[i] : ws == 1 ? (i < 3 ? v[(i + 1) & 3] : 0u) : ws == 2 ? (i < 2 ? v[(i + 2) & 3] : 0u) : (i < 1 ? v[3] : 0u);
+    t[4] = 0u;
+    v4u s;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s[i] = (k & 1) ? __builtin_amdgcn_alignbit(t[i + 1], t[i], 16) : t[i];
+    const v4u z = {0u, 0u, 0u, 0u};
+    return col + 8 <= d ? v : col < d ? s : z;
+}
+
 // Running maximum is only raised when some row of the wave outgrows it by more than this many powers of two;
 // until then probabilities are taken relative to the stale maximum (bounded by 2^kLazyTau, exact in the end
 // because numerator and denominator carry the same factor).  Saves the per-tile rescale of the O accumulators.
@@ -233,19 +260,32 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
         } else {
             // element-wise rows: every load of the row block first, then the zero padding and the packing (written as
             // one chunk after the other, each 2-byte load was waited for before the next was issued)
-            half_t raw[KS][8];
+            if (d >= 8) {
+                v4u raw[KS];
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks)
+                for (int ks = 0; ks < KS; ++ks) raw[ks] = load_chunk_anyalign(qrow, 16 * ks + 8 * g, d);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int c = 16 * ks + 8 * g + e;
-                    raw[ks][e] = qrow[c < d ? c : d - 1];
+                for (int ks = 0; ks < KS; ++ks) {
+                    union { v4u u; v8h h; } t;
+                    t.u = finish_chunk_anyalign(raw[ks], 16 * ks + 8 * g, d);
+                    qf[nb][ks] = t.h;
                 }
-            __builtin_amdgcn_sched_barrier(0);
+            } else {
+                half_t raw[KS][8];
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks)
+                for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-                for (int e = 0; e < 8; ++e) qf[nb][ks][e] = 16 * ks + 8 * g + e < d ? raw[ks][e] : (half_t)0.0f;
+                    for (int e = 0; e < 8; ++e) {
+                        const int c = 16 * ks + 8 * g + e;
+                        raw[ks][e] = qrow[c < d ? c : d - 1];
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) qf[nb][ks][e] = 16 * ks + 8 * g + e < d ? raw[ks][e] : (half_t)0.0f;
+            }
         }
     }
 
@@ -257,52 +297,35 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
         ld_row[x] = cid / CH;
         ld_col[x] = (cid % CH) * 8;
     }
-    // A staged chunk: the 16 bytes as loaded (rows of 16-byte pieces), or its eight elements one per register (element-wise
-    // rows: packed only where the chunk is written to LDS, behind the arithmetic of the current tile; packed where they
-    // are loaded, the loads of the next tile were waited for before that arithmetic began).  Columns >= d hold copies of
-    // the row's last elements (load_chunk_unpadded).
-    // (Only the 32-wide bucket has the registers for it: at 64 it measured -7 %, at 128, which already spills, -16 %.)
-    constexpr bool kPackLate = !kVec && D <= 32;
-    struct Staged {
-        v4u v;
-        uint32_t e[kPackLate ? 8 : 1];
-    };
-    Staged kreg[NLD], vreg[NLD];
-    auto gload = [&](const half_t* __restrict__ base, int tile, Staged (&reg)[NLD]) {
+    // A staged chunk: the 16 bytes as loaded.  For rows of 16-byte pieces they are the chunk (columns >= d hold copies of
+    // the row's last elements: load_chunk_unpadded); for rows at any alignment they become the chunk where it is written
+    // to LDS, behind the arithmetic of the current tile (finish_chunk_anyalign), except that rows of fewer than eight
+    // elements are fetched element by element.
+    v4u kreg[NLD], vreg[NLD];
+    auto gload = [&](const half_t* __restrict__ base, int tile, v4u (&reg)[NLD]) {
         const int kb0 = tile * BC;
 #pragma unroll
         for (int x = 0; x < NLD; ++x) {
             const int r = kb0 + ld_row[x];
             const half_t* __restrict__ rowp = base + (size_t)(r < Nk ? r : Nk - 1) * d;
-            if constexpr (!kPackLate) {
-                reg[x].v = load_chunk_unpadded<kVec, kFullD>(rowp, ld_col[x], d);
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int c = ld_col[x] + e;
-                    reg[x].e[e] = reinterpret_cast<const uint16_t*>(rowp)[c < d ? c : d - 1];
-                }
-            }
+            if constexpr (kVec) reg[x] = load_chunk_unpadded<kVec, kFullD>(rowp, ld_col[x], d);
+            else reg[x] = d >= 8 ? load_chunk_anyalign(rowp, ld_col[x], d) : load_chunk<false, false>(rowp, ld_col[x], d);
         }
     };
-    auto staged_chunk = [&](const Staged& r) {
-        if constexpr (!kPackLate) {
-            return r.v;
-        } else {
-            const v4u p = {r.e[0] | (r.e[1] << 16), r.e[2] | (r.e[3] << 16), r.e[4] | (r.e[5] << 16), r.e[6] | (r.e[7] << 16)};
-            return p;
-        }
+    auto staged_chunk = [&](const v4u& r, int col) {
+        if constexpr (kVec) return r;
+        else return d >= 8 ? finish_chunk_anyalign(r, col, d) : r;
     };
     auto put_k = [&](int buf) {
 #pragma unroll
         for (int x = 0; x < NLD; ++x)
-            *reinterpret_cast<v4u*>(Ks + buf * C::KBUF + ld_row[x] * SK + ld_col[x] * 2) = staged_chunk(kreg[x]);
+            *reinterpret_cast<v4u*>(Ks + buf * C::KBUF + ld_row[x] * SK + ld_col[x] * 2) = staged_chunk(kreg[x], ld_col[x]);
     };
     auto put_v = [&](int buf) {
 #pragma unroll
         for (int x = 0; x < NLD; ++x)
             *reinterpret_cast<v4u*>(Vs + buf * C::VBUF + ld_row[x] * SV +
-                                    ((ld_col[x] * 2) ^ (C::VSWZ ? ((ld_row[x] >> 1) & 1) << 6 : 0))) = staged_chunk(vreg[x]);
+                                    ((ld_col[x] * 2) ^ (C::VSWZ ? ((ld_row[x] >> 1) & 1) << 6 : 0))) = staged_chunk(vreg[x], ld_col[x]);
     };
 
     // ---- direct global -> LDS path: the tile buffers keep their layout (K rows padded by one chunk, V rows with the
@@ -904,7 +927,11 @@ inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
     const int feat = variant & (kVarAlibi | kVarDropout);
     constexpr int AL = kVarAlibi | kVarAlibiLeft;  // ALiBi with no visible key right of its row
     if (!(variant & kVarVec)) {
-        e = launch_fwd_instance<D, NB, ST | kVarAlibi | kVarDropout>(a, st);
+        // rows at any alignment: a plain instance, and one with both features compiled in (slope 0 / threshold 0 make
+        // them identities) for every other request, a non-positive scale among them (its ALiBi step is where the
+        // scores are scaled ahead of the row maximum)
+        e = feat == 0 && a.scale_log2 > 0.0f ? launch_fwd_instance<D, NB, ST>(a, st)
+                                             : launch_fwd_instance<D, NB, ST | kVarAlibi | kVarDropout>(a, st);
     } else if (a.d == D) {
         constexpr int V = ST | kVarVec | kVarFullD;
         const bool kv_once = ST == 0 && a.Tr == 1 && a.kv_group == 1;
