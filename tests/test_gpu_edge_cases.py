@@ -20,15 +20,22 @@ def _slopes(oracle, H):
     return s, torch.from_numpy(s).cuda()
 
 
-# head dims: every bucket edge, multiples of 8 that are not bucket widths, and odd values (element-wise path);
-# 31 is the reference's checked-in head_dim (src/main.cu:42)
-@pytest.mark.parametrize("d", [8, 16, 24, 31, 32, 33, 40, 64, 72, 96, 100, 127, 128])
+# head dims: every bucket edge, multiples of 8 that are not bucket widths, values that are not multiples of 8 (rows at
+# any 2-byte alignment: every length of the partial last chunk, 1 ... 7 elements, in every bucket; below 8, where a row
+# is shorter than a chunk); 31 is the reference's checked-in head_dim (src/main.cu:42).  With ALiBi the other instance
+# of the any-alignment path runs.
+@pytest.mark.parametrize("d", [1, 2, 3, 5, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 24, 31, 32, 33, 40, 41, 47, 60, 63, 64,
+                               65, 72, 77, 90, 95, 96, 97, 100, 106, 119, 125, 127, 128])
 def test_head_dims(fa, oracle, d):
     q, k, v = _qkv(2, 3, 150, 150, d, seed=d)
-    for kw in (dict(), dict(causal=True)):
+    sl, sl_t = _slopes(oracle, 3)
+    for kw, okw in ((dict(), dict()), (dict(causal=True), dict(causal=True)),
+                    (dict(causal=True, alibi_slopes=sl_t), dict(causal=True, slopes=sl))):
+        if "alibi_slopes" in kw and d % 8 == 0 and d not in (8, 128):
+            continue
         o, lse = fa.flash_forward(q, k, v, **kw)
-        O, L = oracle_forward_batched(oracle, q, k, v, **kw)
-        check_o_lse(o, lse, O, L, f"d={d} {kw}")
+        O, L = oracle_forward_batched(oracle, q, k, v, **okw)
+        check_o_lse(o, lse, O, L, f"d={d} {sorted(kw)}")
 
 
 # sequence lengths around the tile sizes (64-key tiles, 128-row groups); 1021 is the reference's checked-in seq_len
