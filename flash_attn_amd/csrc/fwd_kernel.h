@@ -444,6 +444,27 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     auto qk = [&](int buf, v16f (&s)[2][NB]) {
         constexpr bool folded = kFoldAlibi;
         const char* kbase = Ks + buf * C::KBUF + k_rd;
+        if constexpr (folded && NB == 1) {
+            // The first k-step's MFMAs are inline asm here (below), which the issue-order groups at the end of this
+            // function cannot name: with them in the stream the compiler fell back to waiting for every fragment right
+            // behind its request.  So this instance is written out in issue order, fenced step by step: three fragments
+            // ahead, then MFMA and read in turn.
+            constexpr int n = 2 * KS, kAhead = 3;  // step i: k-step i / 2, key block i % 2
+            v8h af[n];
+#pragma unroll
+            for (int i = 0; i < kAhead; ++i) af[i] = *reinterpret_cast<const v8h*>(kbase + (i & 1) * 32 * SK + (i >> 1) * 32);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < n; ++i) {
+                const int ks = i >> 1, kb = i & 1;
+                if (ks == 0) asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(s[kb][0]) : "v"(af[i]), "v"(qf[0][ks]), "v"(calib));
+                else s[kb][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], qf[0][ks], s[kb][0], 0, 0, 0);
+                if (i + kAhead < n)
+                    af[i + kAhead] = *reinterpret_cast<const v8h*>(kbase + ((i + kAhead) & 1) * 32 * SK + ((i + kAhead) >> 1) * 32);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            return;
+        }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
