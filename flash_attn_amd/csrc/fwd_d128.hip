@@ -9,7 +9,9 @@ bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr, long
     // 1024 rows the diagonal, where the waves of a 256-row block run out of keys one after the other, is too large a
     // share of the work (measured 4-9 % slower over B*H = 8 ... 1024 at N = 512 and 1024).  And with one 8-wave
     // work-group per CU its grid should make at least two full rounds of the 256 CUs: below that the 4-wave kernel
-    // (two work-groups of half the rows per CU) fills the chip better (measured +4 ... +13 %, one shape -8 %).
+    // (two work-groups of half the rows per CU) fills the chip better (measured +4 ... +13 %, one shape -8 %) -- except
+    // where an unmasked launch is one round that fills three quarters of the CUs or more (192 ... 256 work-groups:
+    // measured 3-13 % faster with the 8-wave kernel on eleven random shapes of twelve, 128 and fewer 15-35 % slower).
     // The caller's hint (flash_params::kernel_hint: 1 = 4-wave, 2 = 8-wave) overrides these preferences for A/B runs
     // and tests; the 8-wave kernel still needs d == 128 in whole 16-byte rows and more than 128 query rows.
     const bool able = vec && d == 128 && Nq > 128;
@@ -18,7 +20,8 @@ bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr, long
     const bool narrow_window = (wl >= 0 && wl < 512) || (wr >= 0 && wr < 512 && !causal);
     const bool short_causal = causal && Nq <= 1024;
     const long long groups = slices * ((Nq + 255) / 256);
-    return able && !narrow_window && !short_causal && groups >= 512;
+    const bool one_full_round = !causal && wl < 0 && wr < 0 && groups >= 192 && groups <= 256;
+    return able && !narrow_window && !short_causal && (groups >= 512 || one_full_round);
 }
 
 int launch_fwd_d128(const FwdArgs& a, int variant, int nb, hipStream_t st)
