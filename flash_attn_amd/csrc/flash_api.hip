@@ -136,10 +136,10 @@ void fill_args(const flash_params* p, int splits, fa::FwdArgs* a)
 // variant bits of the tiled kernel for p (kVarVec | kVarAlibi | kVarDropout of fwd_kernel.h)
 int tiled_variant(const flash_params* p)
 {
-    // A non-positive scale does not commute with the row maximum: only the element-wise instance scales first.
+    // A non-positive scale does not commute with the row maximum: only the any-alignment instance that serves every request scales first.
     int variant = (p->d % 8 == 0 && p->softmax_scale > 0.0f && !p->scores_out) ? 1 : 0;  // (the score dump lives there too)
     // A dropout probability below 2^-16 has threshold 0 (every element kept, survivors still scaled): the vector
-    // instances apply the decisions with threshold - 1 and leave that case to the element-wise one.
+    // instances apply the decisions with threshold - 1 and leave that case to the same instance.
     if (p->dropout_p > 0.0f && flash_dropout_threshold(p->dropout_p) == 0) variant = 0;
     if (p->alibi_slopes) variant |= 2;
     if (p->dropout_p > 0.0f) variant |= 4;
@@ -196,12 +196,13 @@ int auto_splits_tiled(const flash_params* p, int n_blocks, bool decode = false)
     if (slices * Tr >= 4LL * kNumCU) return 1;  // (the reference's early exit: four rounds of work-groups as they are)
     const int bucket = (p->d + 31) / 32;  // head-dim bucket of the kernel instance: 1 ... 4
     // microseconds per tile of a lone work-group, by bucket; x 1.1 where the tiles are staged through registers
-    // (d % 8 == 0 but not the bucket's width), x 1.5 for rows at any alignment (d % 8 != 0; x 1.15 in the 32-wide bucket)
+    // (d % 8 == 0 but not the bucket's width), x 1.15 for rows at any alignment (d % 8 != 0; measured 1.0-1.2 x the
+    // bucket-wide instance)
     static const float kTile[5] = {0.0f, 0.5f, 0.72f, 0.88f, 1.0f};
     const bool dma = vec && p->d == 32 * bucket;
     // (decode launches, whose tiles no other work-group has asked for before: twice that, and 0.04 us per split for
     // the combine of their few rows; fitted to 55 random decode shapes of the tiled routes)
-    const float b = (pp ? 1.97f : kTile[bucket] * (dma ? 1.0f : vec ? 1.1f : bucket == 1 ? 1.15f : 1.5f)) * (decode ? 2.0f : 1.0f);
+    const float b = (pp ? 1.97f : kTile[bucket] * (dma ? 1.0f : vec ? 1.1f : 1.15f)) * (decode ? 2.0f : 1.0f);
     const float rho2 = pp ? 1.0f : dma ? 1.32f : vec ? 1.35f : 1.4f;
     const float rho3 = (!pp && vec && p->d <= 64) ? rho2 * 1.12f : rho2;  // three places per CU up to d = 64
     // a: prologue + epilogue of a work-group; c0 + c1 s: the combine launch and what every further split adds to it and to
@@ -345,7 +346,7 @@ int scratch_of_current_device(unsigned char** out)
 constexpr int kRouteTiled = 0, kRouteStream = 1;
 int splitkv_route(const flash_params* p, fa::FwdArgs* a)
 {
-    if (p->scores_out) return kRouteTiled;  // debug dump: element-wise instance of the tiled kernel
+    if (p->scores_out) return kRouteTiled;  // debug dump: the tiled kernel's instance that serves every request
     if (p->Nq == 1 && a->kv_group >= 4 && !p->alibi_slopes && a->wl < 0 && p->dropout_p == 0.0f) {
         // Decode with grouped K/V heads: the G query heads of one K/V head, one row each, are the G rows of one
         // attention problem over that K/V head -- Q [B,H,1,d] is [B,H_kv,G,d] in memory, and so are O, LSE and the

@@ -21,7 +21,7 @@
 //    element test.  The KV tile range of the group is pruned like src/flash_forward.h:39-48.
 //  * Ragged Nq / Nk: row indices of loads are clamped, stores are predicated, keys >= Nk are masked (the
 //    reference zero-fills them and leaves them unmasked).  Head dims that are not a multiple of 8 use the
-//    element-wise load / store path (kVec = false).
+//    instances for rows at any alignment (kVec = false).
 #pragma once
 #include <type_traits>
 
@@ -102,29 +102,29 @@ __device__ __forceinline__ v4u load_chunk_unpadded(const half_t* __restrict__ ro
 
 // Rows that start at any 2-byte boundary (d % 8 != 0), d >= 8: a chunk is still one 16-byte load -- the hardware runs in
 // unaligned access mode -- taken at the chunk's own column, or, for the row's last, partial chunk and for chunks past the
-// row, at column d - 8, so that no load ever leaves the row.  finish_chunk_anyalign turns what was loaded into the chunk
-// at column col: whole chunks as they are; the partial one moved down by 8 - d % 8 elements, which brings zeroes in
-// from the top, exactly its columns >= d; chunks past the row zero.  (Two steps, so that the caller can keep the
-// arithmetic away from the load: see load_chunk_unpadded.)  Element by element, a 64 x 32 tile took 16 two-byte loads
-// per thread with an address computation each, where this takes two loads.
+// row, at column d - 8, so that no load ever leaves the row.  Nothing is moved into place afterwards: the last chunk
+// position of a row simply stands for the columns d - 8 ... d - 1 instead of 8 (d / 8) ... 8 (d / 8) + 7.
+//   Q   the columns that the chunk before has covered already (the first 8 - d % 8 of the partial chunk) are zeroed, and so
+//       are chunks past the row (mask_q_chunk_anyalign): every product with them is 0 times finite data of the K row itself.
+//   K   as loaded.
+//   V   as loaded: the chunk position yields O's columns d - 8 ... d - 1, of which the epilogue stores the row's last 16
+//       bytes; chunks past the row yield columns that are never stored.
+// Element by element, a 64 x 32 tile took 16 two-byte loads per thread with an address computation each, where this takes
+// two loads and no arithmetic on the data.
 typedef v4u __attribute__((aligned(2))) v4u_anyalign;
+typedef v4f __attribute__((aligned(4))) v4f_anyalign;
 __device__ __forceinline__ v4u load_chunk_anyalign(const half_t* __restrict__ rowp, int col, int d)
 {
     return *reinterpret_cast<const v4u_anyalign*>(rowp + (col + 8 <= d ? col : d - 8));
 }
-__device__ __forceinline__ v4u finish_chunk_anyalign(v4u v, int col, int d)
+__device__ __forceinline__ v8h mask_q_chunk_anyalign(v4u v, int col, int d)
 {
-    const int k = 8 - (d & 7);  // elements to move down by: the same in every lane, 1 ... 7
-    const int ws = k >> 1;      // whole 32-bit words of it
-    uint32_t t[5];
+    union { v4u u; v8h h; } t;
+    t.u = v;
+    const int covered = col + 8 <= d ? 0 : col < d ? 8 - (d & 7) : 8;  // leading elements that must not count
 #pragma unroll
-    for (int i = 0; i < 4; ++i) t[i] = ws == 0 ? v[i] : ws == 1 ? (i < 3 ? v[(i + 1) & 3] : 0u) : ws == 2 ? (i < 2 ? v[(i + 2) & 3] : 0u) : (i < 1 ? v[3] : 0u);
-    t[4] = 0u;
-    v4u s;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) s[i] = (k & 1) ? __builtin_amdgcn_alignbit(t[i + 1], t[i], 16) : t[i];
-    const v4u z = {0u, 0u, 0u, 0u};
-    return col + 8 <= d ? v : col < d ? s : z;
+    for (int e = 0; e < 8; ++e) t.h[e] = e >= covered ? t.h[e] : (half_t)0.0f;
+    return t.h;
 }
 
 // Running maximum is only raised when some row of the wave outgrows it by more than this many powers of two;
@@ -151,6 +151,12 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     // Instances whose rows are whole 16-byte chunks of exactly D columns fetch their tiles straight into LDS
     // (global_load_lds_dwordx4) instead of through registers: measured +6-12 % at D = 128, +1-4 % at D = 64 and 96.
     constexpr bool kDma = kVec && kFullD;
+    // Rows at any alignment (kVec false) have a plain, an ALiBi and a dropout instance, which count on d >= 8, a positive
+    // scale, a slope table where ALiBi is compiled in and a dropout threshold of at least 1 like the vector instances
+    // do, and one instance with both features compiled in that serves every request (kEvery: slope 0 / threshold 0
+    // make the features identities), a non-positive scale, rows of fewer than eight elements and the score dump
+    // among them.
+    constexpr bool kEvery = !kVec && kAlibi && kDropout;
     constexpr int NSTG = kDma ? C::NSTG : 2;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     char* const Ks = smem;
@@ -258,18 +264,16 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                 qf[nb][ks] = t.h;
             }
         } else {
-            // element-wise rows: every load of the row block first, then the zero padding and the packing (written as
+            // rows at any alignment: every load of the row block first, then the zero padding and the packing (written as
             // one chunk after the other, each 2-byte load was waited for before the next was issued)
-            if (d >= 8) {
+            if (!kEvery || d >= 8) {
                 v4u raw[KS];
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) raw[ks] = load_chunk_anyalign(qrow, 16 * ks + 8 * g, d);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    union { v4u u; v8h h; } t;
-                    t.u = finish_chunk_anyalign(raw[ks], 16 * ks + 8 * g, d);
-                    qf[nb][ks] = t.h;
+                    qf[nb][ks] = mask_q_chunk_anyalign(raw[ks], 16 * ks + 8 * g, d);
                 }
             } else {
                 half_t raw[KS][8];
@@ -297,10 +301,9 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
         ld_row[x] = cid / CH;
         ld_col[x] = (cid % CH) * 8;
     }
-    // A staged chunk: the 16 bytes as loaded.  For rows of 16-byte pieces they are the chunk (columns >= d hold copies of
-    // the row's last elements: load_chunk_unpadded); for rows at any alignment they become the chunk where it is written
-    // to LDS, behind the arithmetic of the current tile (finish_chunk_anyalign), except that rows of fewer than eight
-    // elements are fetched element by element.
+    // A staged chunk: the 16 bytes as loaded (chunk positions past the row's whole chunks hold the row's last elements:
+    // load_chunk_unpadded, load_chunk_anyalign), except that rows of fewer than eight elements are fetched element by
+    // element and padded with zeroes.
     v4u kreg[NLD], vreg[NLD];
     auto gload = [&](const half_t* __restrict__ base, int tile, v4u (&reg)[NLD]) {
         const int kb0 = tile * BC;
@@ -309,23 +312,19 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
             const int r = kb0 + ld_row[x];
             const half_t* __restrict__ rowp = base + (size_t)(r < Nk ? r : Nk - 1) * d;
             if constexpr (kVec) reg[x] = load_chunk_unpadded<kVec, kFullD>(rowp, ld_col[x], d);
-            else reg[x] = d >= 8 ? load_chunk_anyalign(rowp, ld_col[x], d) : load_chunk<false, false>(rowp, ld_col[x], d);
+            else reg[x] = !kEvery || d >= 8 ? load_chunk_anyalign(rowp, ld_col[x], d) : load_chunk<false, false>(rowp, ld_col[x], d);
         }
-    };
-    auto staged_chunk = [&](const v4u& r, int col) {
-        if constexpr (kVec) return r;
-        else return d >= 8 ? finish_chunk_anyalign(r, col, d) : r;
     };
     auto put_k = [&](int buf) {
 #pragma unroll
         for (int x = 0; x < NLD; ++x)
-            *reinterpret_cast<v4u*>(Ks + buf * C::KBUF + ld_row[x] * SK + ld_col[x] * 2) = staged_chunk(kreg[x], ld_col[x]);
+            *reinterpret_cast<v4u*>(Ks + buf * C::KBUF + ld_row[x] * SK + ld_col[x] * 2) = kreg[x];
     };
     auto put_v = [&](int buf) {
 #pragma unroll
         for (int x = 0; x < NLD; ++x)
             *reinterpret_cast<v4u*>(Vs + buf * C::VBUF + ld_row[x] * SV +
-                                    ((ld_col[x] * 2) ^ (C::VSWZ ? ((ld_row[x] >> 1) & 1) << 6 : 0))) = staged_chunk(vreg[x], ld_col[x]);
+                                    ((ld_col[x] * 2) ^ (C::VSWZ ? ((ld_row[x] >> 1) & 1) << 6 : 0))) = vreg[x];
     };
 
     // ---- direct global -> LDS path: the tile buffers keep their layout (K rows padded by one chunk, V rows with the
@@ -408,10 +407,10 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
 
     // Scores leave the MFMA unscaled.  With a positive scale the scaling commutes with the row maximum and is folded
     // into the exponent (one fma per score): cs = scale, and the ALiBi bias is added beforehand divided by the scale.
-    // A non-positive scale is served by the element-wise instance alone (the host sends it there): then the scores are
+    // A non-positive scale is served by the kEvery instance alone (the host sends it there): then the scores are
     // scaled first and cs = 1.
     const float c2 = a.scale_log2;
-    const bool scale_late = kVec || c2 > 0.0f;
+    const bool scale_late = !kEvery || c2 > 0.0f;
     const float cs = scale_late ? c2 : 1.0f;
     // The ALiBi slope of the head is read once the first tile requests are on their way (read_slope below): it is a
     // vector load, the wait for it counts every older request as well, and nothing before the first softmax needs it.
@@ -425,8 +424,8 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     v16f calib;
     auto read_slope = [&]() {
         if constexpr (kAlibi) {
-            // (the vector instances are only launched with a slope table; the element-wise one serves every request)
-            slope2 = (kVec || a.alibi) ? a.alibi[h] * kLog2e : 0.0f;
+            // (only the kEvery instance is launched without a slope table)
+            slope2 = (!kEvery || a.alibi) ? a.alibi[h] * kLog2e : 0.0f;
             nsig = scale_late ? -slope2 / c2 : 0.0f;
             if constexpr (kFoldAlibi) {
 #pragma unroll
@@ -569,7 +568,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                     }
                 }
             }
-            if constexpr (!kVec) {
+            if constexpr (kEvery) {
                 if (a.scores_out != nullptr && row_i[nb] < Nq) {  // debug dump of the visible scores, natural-log units
                     float* srow = a.scores_out + ((size_t)bh * Nq + row_i[nb]) * Nk;
                     const float unit = (scale_late ? cs : 1.0f) * kLn2;
@@ -637,7 +636,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                         // the lane's eight keys among the 16 from jg on: field f belongs to key jg + 8*(f>>2) + 4*g + (f&3)
                         const int jg = kb0 + 32 * kb + 16 * q;
                         const v4u w = philox4x32_10_c2(dropout_call((uint32_t)(jg + 4 * g)), i_u, bh_hi, bh_lo, a.off_lo, a.seed_lo, a.seed_hi);
-                        if constexpr (kVec) {
+                        if constexpr (!kEvery) {
                             // registers 8q + 2k and 8q + 2k + 1 become one packed fp16 word, fields 2k and 2k + 1 are the
                             // halves of Philox word k: the decisions are applied to the packed word (keep_pair)
 #pragma unroll
@@ -664,7 +663,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                         }
                     }
             }
-            if constexpr (!(kDropout && kVec)) {  // (there the dropout step has packed them already)
+            if constexpr (!(kDropout && !kEvery)) {  // (there the dropout step has packed them already)
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -815,6 +814,14 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                                      oacc[mb][nb][4 * rg + 2] * inv, oacc[mb][nb][4 * rg + 3] * inv};
                             *reinterpret_cast<v4f*>(op + dc) = o;
                         }
+                    } else if (!kEvery || d >= 8) {
+                        // rows at any alignment: the chunk position behind the row's whole chunks holds columns d - 8 ... d - 1
+                        const int c0 = d & ~7, rem = d & 7;
+                        if (dc < c0 || (rem != 0 && dc < c0 + 8)) {
+                            v4f o = {oacc[mb][nb][4 * rg] * inv, oacc[mb][nb][4 * rg + 1] * inv,
+                                     oacc[mb][nb][4 * rg + 2] * inv, oacc[mb][nb][4 * rg + 3] * inv};
+                            *reinterpret_cast<v4f_anyalign*>(op + (dc < c0 ? dc : dc - (8 - rem))) = o;
+                        }
                     } else {
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
@@ -823,7 +830,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                 }
         } else {
             if (g == 0) a.LSE[(size_t)bh * Nq + i] = lse;
-            if constexpr (!kVec) {
+            if (kEvery && d < 8) {
                 half_t* op = a.O + ((size_t)bh * Nq + i) * d;
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
@@ -837,9 +844,9 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
             }
         }
     }
-    if constexpr (kVec) {
+    if (!kEvery || d >= 8) {
         if (a.num_splits == 1) {
-            // O of the vector path: a lane holds 4 consecutive head-dim columns of one row at a time, which as a direct
+            // A lane holds 4 consecutive head-dim columns of one row at a time, which as a direct
             // store would be 32 rows x 8 bytes per instruction.  The wave's 32 x d block goes through LDS instead (the tile
             // buffers are free behind the last barrier; rows padded by 16 bytes) and leaves in consecutive 16-byte pieces
             // of whole rows.  The stores are non-temporal: O is not read again by this launch, and lines left dirty in L2
@@ -867,9 +874,13 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
                 const int p = p0 + lane;
                 const int rl = p / CH, ch = p % CH;
                 const int gi = q0 + wave * C::RW + rl;
-                if (p < NP && gi < Nq && (kFullD || ch * 8 < d))
-                    __builtin_nontemporal_store(*reinterpret_cast<const v4u*>(ost + rl * SO + ch * 16),
-                                                reinterpret_cast<v4u*>(Ob + (size_t)gi * d * 2 + ch * 16));
+                if (p < NP && gi < Nq && (kFullD || ch * 8 < d)) {
+                    const v4u piece = *reinterpret_cast<const v4u*>(ost + rl * SO + ch * 16);
+                    if constexpr (kVec)
+                        __builtin_nontemporal_store(piece, reinterpret_cast<v4u*>(Ob + (size_t)gi * d * 2 + ch * 16));
+                    else  // rows at any alignment: the last chunk position holds the row's last 16 bytes
+                        __builtin_nontemporal_store(piece, reinterpret_cast<v4u_anyalign*>(Ob + (size_t)gi * d * 2 + (ch * 8 + 8 <= d ? ch * 16 : (d - 8) * 2)));
+                }
             }
         }
     }
@@ -939,8 +950,8 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
 }
 
 // The instances of a bucket: {d == bucket, d % 8 == 0} x {plain, ALiBi, ALiBi with every visible key at or left of its
-// row, dropout, both}, and the element-wise path with both features compiled in (slope 0 / threshold 0 make them identities, so it serves every request
-// with d % 8 != 0).  ST = kVarStamp selects their instrumented twins (debug time stamps).
+// row, dropout, both}, and for rows at any alignment (d % 8 != 0) {plain, ALiBi, dropout, both}, the last of which serves
+// every other request as well.  ST = kVarStamp selects their instrumented twins (debug time stamps).
 template <int D, int NB, int ST>
 inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
 {
@@ -948,11 +959,16 @@ inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
     const int feat = variant & (kVarAlibi | kVarDropout);
     constexpr int AL = kVarAlibi | kVarAlibiLeft;  // ALiBi with no visible key right of its row
     if (!(variant & kVarVec)) {
-        // rows at any alignment: a plain instance, and one with both features compiled in (slope 0 / threshold 0 make
-        // them identities) for every other request, a non-positive scale among them (its ALiBi step is where the
-        // scores are scaled ahead of the row maximum)
-        e = feat == 0 && a.scale_log2 > 0.0f ? launch_fwd_instance<D, NB, ST>(a, st)
-                                             : launch_fwd_instance<D, NB, ST | kVarAlibi | kVarDropout>(a, st);
+        // rows at any alignment: a plain, an ALiBi and a dropout instance, and one with both features compiled in
+        // (slope 0 / threshold 0 make them identities) for every other request: both features at once, a non-positive
+        // scale (its ALiBi step is where the scores are scaled ahead of the row maximum), the score dump, rows of
+        // fewer than eight elements, a dropout threshold of 0
+        const bool every = feat == (kVarAlibi | kVarDropout) || a.scale_log2 <= 0.0f || a.scores_out != nullptr || a.d < 8 ||
+                           (feat == kVarDropout && a.drop_thr == 0);
+        if (every) e = launch_fwd_instance<D, NB, ST | kVarAlibi | kVarDropout>(a, st);
+        else if (feat == 0) e = launch_fwd_instance<D, NB, ST>(a, st);
+        else if (feat == kVarAlibi) e = launch_fwd_instance<D, NB, ST | kVarAlibi>(a, st);
+        else e = launch_fwd_instance<D, NB, ST | kVarDropout>(a, st);
     } else if (a.d == D) {
         constexpr int V = ST | kVarVec | kVarFullD;
         const bool kv_once = ST == 0 && a.Tr == 1 && a.kv_group == 1;

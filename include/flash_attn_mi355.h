@@ -90,7 +90,7 @@ typedef struct flash_params {
      * softmax_scale * q_i.k_j - slope_h * |i - j| in fp32, for every (i, j) that the masks leave visible, into
      * scores_out [B,H,Nq,Nk]; entries of masked pairs are not written (fill the buffer with -inf beforehand to read it
      * as the masked score matrix).  The call then takes the one kernel instance that serves every
-     * feature and head dim, which is up to twice as slow.  No counterpart in the reference. */
+     * feature and head dim, which is about 20 % slower.  No counterpart in the reference. */
     float *scores_out;
     /* Which tiled kernel serves the call, for A/B measurements and tests: 0 = the library chooses (by shape),
      * 1 = the 4-wave kernel (128 query rows per work-group), 2 = the 8-wave ping-pong kernel (256 rows; needs d == 128

@@ -22,8 +22,8 @@ def _slopes(oracle, H):
 
 # head dims: every bucket edge, multiples of 8 that are not bucket widths, values that are not multiples of 8 (rows at
 # any 2-byte alignment: every length of the partial last chunk, 1 ... 7 elements, in every bucket; below 8, where a row
-# is shorter than a chunk); 31 is the reference's checked-in head_dim (src/main.cu:42).  With ALiBi the other instance
-# of the any-alignment path runs.
+# is shorter than a chunk, served by the any-alignment instance that serves every request); 31 is the reference's
+# checked-in head_dim (src/main.cu:42).  With ALiBi the ALiBi instance of the any-alignment path runs.
 @pytest.mark.parametrize("d", [1, 2, 3, 5, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 24, 31, 32, 33, 40, 41, 47, 60, 63, 64,
                                65, 72, 77, 90, 95, 96, 97, 100, 106, 119, 125, 127, 128])
 def test_head_dims(fa, oracle, d):
@@ -36,6 +36,41 @@ def test_head_dims(fa, oracle, d):
         o, lse = fa.flash_forward(q, k, v, **kw)
         O, L = oracle_forward_batched(oracle, q, k, v, **okw)
         check_o_lse(o, lse, O, L, f"d={d} {sorted(kw)}")
+
+
+# Rows at any alignment have four kernel instances per bucket: plain, ALiBi, dropout, and the one that serves every other
+# request (both features at once, dropout thresholds of 0, non-positive scales).  Each is run on every length of the
+# partial last chunk, unsplit (O leaves as the row's whole chunks plus its last 16 bytes) and in three splits (fp32
+# partial rows, 4-byte aligned), with the keep decisions dumped where dropout is on; a threshold of 1 is the smallest the
+# dropout instance's packed decisions see.
+@pytest.mark.parametrize("d", [9, 12, 15, 17, 27, 31, 34, 45, 62, 63, 67, 76, 93, 99, 100, 105, 110, 123, 127])
+def test_any_alignment_instances(fa, oracle, d):
+    import torch
+    B, H, Nq, Nk = 1, 3, 135, 203
+    q, k, v = _qkv(B, H, Nq, Nk, d, seed=1000 + d)
+    sl, sl_t = _slopes(oracle, H)
+    p_of = {"dropout": 0.3, "dropout_thr1": 2.0 ** -16, "dropout_thr0": 1e-6}
+    for feat in ("plain", "alibi", "dropout", "dropout_thr1", "both", "dropout_thr0", "negative_scale"):
+        kw, okw = dict(causal=True), dict(causal=True)
+        if feat in ("alibi", "both"):
+            kw["alibi_slopes"], okw["slopes"] = sl_t, sl
+        if feat == "negative_scale":
+            kw["softmax_scale"], okw["scale"] = -0.2, -0.2
+        p = p_of.get(feat, 0.3 if feat == "both" else 0.0)
+        if p > 0.0:
+            keep = oracle.dropout_keep_mask(77, d, p, B, H, Nq, Nk)
+            kw.update(dropout_p=p, seed=77, offset=d)
+            okw.update(keep_mask=torch.from_numpy(keep), p_drop=p)
+        O, L = oracle_forward_batched(oracle, q, k, v, **okw)
+        if p > 0.0:
+            o, lse, km = fa.flash_forward(q, k, v, return_keep_mask=True, **kw)
+            vis = np.tril(np.ones((Nq, Nk), dtype=bool), k=Nk - Nq)
+            assert np.array_equal(km.cpu().numpy()[..., vis], keep[..., vis]), f"d={d} {feat}"
+        else:
+            o, lse = fa.flash_forward(q, k, v, **kw)
+        check_o_lse(o, lse, O, L, f"d={d} {feat}")
+        o3, lse3 = fa.flash_forward_splitkv(q, k, v, num_splits=3, **kw)
+        check_o_lse(o3, lse3, O, L, f"d={d} {feat} three splits")
 
 
 # sequence lengths around the tile sizes (64-key tiles, 128-row groups); 1021 is the reference's checked-in seq_len
@@ -151,7 +186,7 @@ def test_dropout_mask_bit_exact_and_output(fa, oracle, shape):
 @pytest.mark.parametrize("shape", [(1, 2, 300, 300, 128), (1, 2, 150, 150, 64)])
 def test_dropout_threshold_edges(fa, oracle, shape):
     """The smallest thresholds: p below 2^-16 has threshold 0 (every element kept, survivors still scaled by 1/(1-p)) and
-    is served by the element-wise instance; p = 2^-16 has threshold 1, the smallest one the vector instances' packed
+    is served by the any-alignment instance that serves every request; p = 2^-16 has threshold 1, the smallest one the vector instances' packed
     keep decisions (saturating subtraction of threshold - 1) see; p close to 1 the largest."""
     import torch
     B, H, Nq, Nk, d = shape
@@ -282,7 +317,7 @@ def test_splitkv_heuristic_and_decode_variants(fa, oracle):
 @pytest.mark.parametrize("H,Hk,Nq,Nk,d,kw", [
     (8, 2, 300, 300, 128, dict(causal=True)),       # 8-wave kernel
     (6, 3, 200, 333, 64, dict()),                    # 4-wave kernel, Nq != Nk
-    (4, 1, 129, 129, 31, dict(window=(40, 10))),     # multi-query, element-wise head dim
+    (4, 1, 129, 129, 31, dict(window=(40, 10))),     # multi-query, head dim at any alignment
     (8, 4, 64, 500, 96, dict(causal=True)),
     # slice counts that are multiples of 8 x (query heads per K/V head): the slice order keeps the heads of a K/V head
     # on one XCD (a permutation of the slices inside a chunk, in both tiled kernels and in split mode)
@@ -357,7 +392,7 @@ def test_decode_routes_times_masks(fa, oracle, G, window, causal):
     for extra in (dict(), dict(dropout_p=0.0, softmax_scale=d ** -0.5)):
         o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=4, window=window, causal=causal, **extra)
         check_o_lse(o, lse, O, L, f"decode G={G} window={window} causal={causal}")
-    # the element-wise tiled fallback (odd head dim) under the same masks
+    # the tiled fallback for rows at any alignment (odd head dim) under the same masks
     q2, k2, v2 = q[..., :31].contiguous(), k[..., :31].contiguous(), v[..., :31].contiguous()
     O2, L2 = oracle_forward_batched(oracle, q2, k2.repeat_interleave(G, dim=1), v2.repeat_interleave(G, dim=1),
                                     window=window, causal=causal)
@@ -386,7 +421,7 @@ def test_unbounded_windows_written_as_large_numbers(fa):
     (2, 600, 128, dict(causal=True)),                 # 8-wave kernel
     (1, 600, 128, dict(causal=True)),                 # 4-wave kernel, tiles fetched straight into LDS
     (0, 300, 64, dict(window=(100, 0))),              # 4-wave kernel, register-staged tiles
-    (0, 150, 31, dict()),                             # element-wise instance
+    (0, 150, 31, dict()),                             # any-alignment instance
 ])
 def test_stage_stamps(fa, oracle, hint, N, d, kw):
     """Debug output: per work-group stamps of the constant 100 MHz counter are non-decreasing from stage to stage, the
