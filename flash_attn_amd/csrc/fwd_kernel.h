@@ -137,10 +137,19 @@ constexpr float kLazyTau = 8.0f;
 // (causal mask or a right window of 0), which lets the bias ride in the MFMA accumulator (see calib below).
 // kVarKvOnce (with kVarVec, kVarFullD, no other feature): every K/V tile is requested by this work-group alone -- one row
 // block per slice and one query head per K/V head, the shape of a decode launch -- and its requests are non-temporal.
-constexpr int kVarVec = 1, kVarAlibi = 2, kVarDropout = 4, kVarFullD = 8, kVarStamp = 16, kVarAlibiLeft = 32, kVarKvOnce = 64;
+// kVarEvery (with kVarAlibi and kVarDropout, without kVarVec): the instance that serves every request, see kEvery below.
+constexpr int kVarVec = 1, kVarAlibi = 2, kVarDropout = 4, kVarFullD = 8, kVarStamp = 16, kVarAlibiLeft = 32, kVarKvOnce = 64,
+              kVarEvery = 128;
+
+// work-groups per CU: three up to D = 64 (168 VGPRs), except for the instance that serves every request, which stages
+// its tiles through registers
+constexpr int fwd_groups_per_cu(int D, int NB, int VAR)
+{
+    return NB == 1 ? (D <= 64 && (VAR & kVarEvery) == 0 ? 3 : 2) : 1;
+}
 
 template <int D, int NB, int VAR>
-__global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 0 ? 3 : 2) : 1) fwd_kernel(const FwdArgs a)
+__global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel(const FwdArgs a)
 {
     constexpr bool kVec = (VAR & kVarVec) != 0, kAlibi = (VAR & kVarAlibi) != 0, kDropout = (VAR & kVarDropout) != 0,
                    kFullD = (VAR & kVarFullD) != 0, kStamp = (VAR & kVarStamp) != 0, kKvOnce = (VAR & kVarKvOnce) != 0;
@@ -148,15 +157,18 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     Stamps<kStamp> stamps;
     stamps.take(0);
     constexpr int BC = C::BC, KS = C::KS, MB = C::MB, CH = C::CH, SK = C::SK, SV = C::SV, NLD = C::NLD;
-    // Instances whose rows are whole 16-byte chunks of exactly D columns fetch their tiles straight into LDS
-    // (global_load_lds_dwordx4) instead of through registers: measured +6-12 % at D = 128, +1-4 % at D = 64 and 96.
-    constexpr bool kDma = kVec && kFullD;
-    // Rows at any alignment (kVec false) have a plain, an ALiBi and a dropout instance, which count on d >= 8, a positive
-    // scale, a slope table where ALiBi is compiled in and a dropout threshold of at least 1 like the vector instances
-    // do, and one instance with both features compiled in that serves every request (kEvery: slope 0 / threshold 0
-    // make the features identities), a non-positive scale, rows of fewer than eight elements and the score dump
-    // among them.
-    constexpr bool kEvery = !kVec && kAlibi && kDropout;
+    // Tiles go from global memory straight into LDS (global_load_lds_dwordx4) instead of through registers: measured
+    // +6-12 % at D = 128, +1-4 % at D = 64 and 96.  The request takes global addresses at any 2-byte boundary, so rows of
+    // any length from eight elements on are served; only the instance that also serves shorter rows stages through
+    // registers (kEvery, defined below).
+    constexpr bool kDma = (VAR & kVarEvery) == 0;
+    // Rows at any alignment (kVec false) have the same four instances as rows of whole chunks: plain, ALiBi, dropout, both.
+    // They count on d >= 8, a positive scale, a slope table where ALiBi is compiled in and a dropout threshold of at least
+    // 1 like the vector instances do.  One more instance, with both features compiled in, serves every request (kEvery:
+    // slope 0 / threshold 0 make the features identities), a non-positive scale, rows of fewer than eight elements and
+    // the score dump among them.
+    constexpr bool kEvery = (VAR & kVarEvery) != 0;
+    static_assert(!kEvery || (!kVec && kAlibi && kDropout), "the instance that serves every request");
     constexpr int NSTG = kDma ? C::NSTG : 2;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     char* const Ks = smem;
@@ -331,6 +343,10 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
     // 64-byte halves exchanged in rows 2, 3 mod 4), and a request fills 64 consecutive 16-byte chunks of a buffer: lane l of
     // block x fetches whatever belongs into chunk 64 x + l (the pad chunk of a K row gets a copy of its neighbour).
     // Blocks go round the four waves; the odd K block goes to the waves that still have a block index left for it.
+    // Rows shorter than the bucket: chunk positions past the row's whole chunks fetch the row's last 16 bytes (see
+    // load_chunk_unpadded, load_chunk_anyalign).
+    const int row_bytes = kFullD ? D * 2 : d * 2;
+    auto chunk_offset = [&](int c) { return kFullD ? c * 16 : (c * 8 + 8 <= d ? c * 16 : (d - 8) * 2); };
     uint32_t koff[C::NKX], voff[C::NVX];
     int krow[C::NKX], vrow[C::NVX];
     if constexpr (kDma) {
@@ -339,14 +355,14 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
             const int q = 64 * (wave + 4 * i) + lane;
             krow[i] = q / (CH + 1);
             const int col = q % (CH + 1);
-            koff[i] = (uint32_t)(krow[i] * D * 2 + (col < CH ? col : CH - 1) * 16);
+            koff[i] = (uint32_t)(krow[i] * row_bytes + chunk_offset(col < CH ? col : CH - 1));
         }
 #pragma unroll
         for (int i = 0; i < C::NVX; ++i) {
             const int q = 64 * (wave + 4 * i) + lane;
             vrow[i] = q / CH;
             const int c = q % CH;
-            voff[i] = (uint32_t)(vrow[i] * D * 2 + (C::VSWZ ? c ^ (((vrow[i] >> 1) & 1) << 2) : c) * 16);
+            voff[i] = (uint32_t)(vrow[i] * row_bytes + chunk_offset(C::VSWZ ? c ^ (((vrow[i] >> 1) & 1) << 2) : c));
         }
     }
     const bool k_extra = wave + 4 * (C::NKX - 1) <= CH;  // the last round of K blocks exists for this wave
@@ -354,7 +370,7 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
         // The tile's offset joins the scalar base address, so that a request of a whole tile needs no vector
         // arithmetic at all; only the last tile of a ragged sequence adjusts rows: keys past Nk re-read key Nk - 1
         // (their scores are masked).
-        const size_t tb = (size_t)tile * (size_t)(BC * D * 2);
+        const size_t tb = (size_t)tile * (size_t)(BC * row_bytes);
         const int rows_left = Nk - tile * BC;  // >= 1
         FA_LDS char* const kst = (FA_LDS char*)smem + stage * C::KBUF;
         FA_LDS char* const vst = (FA_LDS char*)smem + NSTG * C::KBUF + stage * C::VBUF;
@@ -370,14 +386,14 @@ __global__ void __launch_bounds__(256, NB == 1 ? (D <= 64 && (VAR & kVarVec) != 
             for (int i = 0; i < C::NKX; ++i) {
                 if (i == C::NKX - 1 && !k_extra) break;
                 uint32_t o = koff[i];
-                if (kRagged && krow[i] >= rows_left) o -= (uint32_t)((krow[i] - rows_left + 1) * D * 2);
+                if (kRagged && krow[i] >= rows_left) o -= (uint32_t)((krow[i] - rows_left + 1) * row_bytes);
                 if constexpr (kKvOnce) dma_kib_nt(Kb, o, kst + (wave + 4 * i) * 1024);
                 else dma_kib(Kb, o, kst + (wave + 4 * i) * 1024);
             }
 #pragma unroll
             for (int i = 0; i < C::NVX; ++i) {
                 uint32_t o = voff[i];
-                if (kRagged && vrow[i] >= rows_left) o -= (uint32_t)((vrow[i] - rows_left + 1) * D * 2);
+                if (kRagged && vrow[i] >= rows_left) o -= (uint32_t)((vrow[i] - rows_left + 1) * row_bytes);
                 if constexpr (kKvOnce) dma_kib_nt(Vb, o, vst + (wave + 4 * i) * 1024);
                 else dma_kib(Vb, o, vst + (wave + 4 * i) * 1024);
             }
@@ -942,7 +958,7 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
     if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, attr_done); e != hipSuccess) return e;
     const long long groups = (long long)a.Tr * a.B * a.H * a.num_splits;
     FwdArgs b = a;
-    constexpr int kResident = (NB == 1 && D <= 64 && (VAR & kVarVec) != 0 ? 3 : 2) * kNumCus;
+    constexpr int kResident = (NB == 1 ? fwd_groups_per_cu(D, NB, VAR) : 2) * kNumCus;
     set_slice_order(b, a.Tr * a.num_splits, kResident);
     b.split_rotate = split_rotate_for(b.num_splits, b.slice_chunk);
     b.snake_end = snake_end_for(groups, kResident);
@@ -950,8 +966,8 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
 }
 
 // The instances of a bucket: {d == bucket, d % 8 == 0} x {plain, ALiBi, ALiBi with every visible key at or left of its
-// row, dropout, both}, and for rows at any alignment (d % 8 != 0) {plain, ALiBi, dropout, both}, the last of which serves
-// every other request as well.  ST = kVarStamp selects their instrumented twins (debug time stamps).
+// row, dropout, both}, for rows at any alignment (d % 8 != 0) {plain, ALiBi, dropout, both}, and the one that serves
+// every other request.  ST = kVarStamp selects their instrumented twins (debug time stamps).
 template <int D, int NB, int ST>
 inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
 {
@@ -959,16 +975,16 @@ inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
     const int feat = variant & (kVarAlibi | kVarDropout);
     constexpr int AL = kVarAlibi | kVarAlibiLeft;  // ALiBi with no visible key right of its row
     if (!(variant & kVarVec)) {
-        // rows at any alignment: a plain, an ALiBi and a dropout instance, and one with both features compiled in
-        // (slope 0 / threshold 0 make them identities) for every other request: both features at once, a non-positive
-        // scale (its ALiBi step is where the scores are scaled ahead of the row maximum), the score dump, rows of
-        // fewer than eight elements, a dropout threshold of 0
-        const bool every = feat == (kVarAlibi | kVarDropout) || a.scale_log2 <= 0.0f || a.scores_out != nullptr || a.d < 8 ||
-                           (feat == kVarDropout && a.drop_thr == 0);
-        if (every) e = launch_fwd_instance<D, NB, ST | kVarAlibi | kVarDropout>(a, st);
+        // rows at any alignment: plain, ALiBi, dropout, both, and one more with both features compiled in (slope 0 /
+        // threshold 0 make them identities) for every other request: a non-positive scale (its ALiBi step is where the
+        // scores are scaled ahead of the row maximum), the score dump, rows of fewer than eight elements, a dropout
+        // threshold of 0
+        const bool every = a.scale_log2 <= 0.0f || a.scores_out != nullptr || a.d < 8 || ((feat & kVarDropout) && a.drop_thr == 0);
+        if (every) e = launch_fwd_instance<D, NB, ST | kVarAlibi | kVarDropout | kVarEvery>(a, st);
         else if (feat == 0) e = launch_fwd_instance<D, NB, ST>(a, st);
         else if (feat == kVarAlibi) e = launch_fwd_instance<D, NB, ST | kVarAlibi>(a, st);
-        else e = launch_fwd_instance<D, NB, ST | kVarDropout>(a, st);
+        else if (feat == kVarDropout) e = launch_fwd_instance<D, NB, ST | kVarDropout>(a, st);
+        else e = launch_fwd_instance<D, NB, ST | kVarAlibi | kVarDropout>(a, st);
     } else if (a.d == D) {
         constexpr int V = ST | kVarVec | kVarFullD;
         const bool kv_once = ST == 0 && a.Tr == 1 && a.kv_group == 1;

@@ -132,10 +132,12 @@ def test_split_resolution_and_workspace(fa):
     assert fa.workspace_bytes(1, 1, 128, 128, 64, 8) == (0, 0)
     # automatic choice (num_splits <= 0) for Nq > 1: the count with the lowest estimated time (work-groups on the fullest
     # CU, prologue / epilogue per work-group, partial results per split).  The reference's checked-in shape
-    # B=1,H=8,N=1021 splits 4 ways (64 row blocks -> 256 work-groups), twice that batch stays whole (128 work-groups of
-    # eight tiles measured 19.6 us, 4 splits 26.2), the prefill benchmark shapes stay unsplit
-    assert fa.resolve_splits(1, 8, 1021, 1021, 31, 0) == 4
+    # B=1,H=8,N=1021,d=31 stays whole (64 work-groups of 16 short tiles: measured 14.4 us, 4 splits 16.3), and so does
+    # twice that batch (14.4 us, 4 splits 22.0); half as many slices of twice the length split 4 ways (22.5 us, whole
+    # 29.6); the prefill benchmark shapes stay unsplit
+    assert fa.resolve_splits(1, 8, 1021, 1021, 31, 0) == 1
     assert fa.resolve_splits(2, 8, 1021, 1021, 31, 0) == 1
+    assert fa.resolve_splits(1, 4, 2048, 2048, 63, 0) == 4
     assert fa.resolve_splits(4, 16, 2048, 2048, 128, 0) == 1
     assert fa.resolve_splits(4, 16, 2048, 2048, 128, 0, causal=True) == 1
     assert fa.resolve_splits(8, 32, 1000, 1000, 96, 0, causal=True) == 1

@@ -94,7 +94,8 @@ def _check(out):
 @pytest.mark.parametrize(
     "args",
     [
-        (),  # the reference's own configuration: B1 H8 N1021 d31, split by the heuristic, ragged N and d
+        (),  # the reference's own configuration: B1 H8 N1021 d31, split count from the library's rule, ragged N and d
+        ("--splits", "4"),  # the same in four splits, the count the reference's rule takes
         ("--causal",),
         ("--window", "128"),
         ("--alibi",),
@@ -102,7 +103,7 @@ def _check(out):
         ("--batch", "2", "--heads", "4", "--seq", "640", "--head-dim", "128", "--causal"),
         ("--batch", "2", "--heads", "4", "--seq", "512", "--head-dim", "64", "--fill", "normal", "--tol", "1e9"),
     ],
-    ids=["reference_default", "causal", "window128", "alibi", "causal_nosplit", "d128_causal", "normal_fill"],
+    ids=["reference_default", "reference_default_4_splits", "causal", "window128", "alibi", "causal_nosplit", "d128_causal", "normal_fill"],
 )
 def test_driver_reference_compatible_runs(args):
     r = _run("--iters", "5", *args)
