@@ -62,6 +62,42 @@ struct FwdArgs {
 
 __device__ __forceinline__ int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
+// A work-group whose rows see no key at all (rows above a causal diagonal that starts below them, a split of the key
+// range beyond their mask): O = 0 and LSE = -inf for rows [r0, r1) of head slice bh, or the same in the slice's partial
+// results of split `split`.  The rows are one contiguous piece of memory; it is filled with 16-byte stores at whatever
+// alignment the piece has, the last one ending with the piece.  Called by every thread of the group, before anything else
+// is requested: such a group is done in the time of its stores.
+__device__ __forceinline__ void store_empty_rows(const FwdArgs& a, int bh, int split, int r0, int r1, int tid, int nthreads)
+{
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    typedef u4 __attribute__((aligned(2))) u4_anyalign;
+    char* base;
+    float* lse;
+    size_t bytes;
+    if (a.num_splits > 1) {
+        const size_t prow = ((size_t)bh * a.num_splits + split) * a.Nq + r0;
+        base = reinterpret_cast<char*>(a.O_partial + prow * a.d);
+        lse = a.LSE_partial + prow;
+        bytes = (size_t)(r1 - r0) * a.d * sizeof(float);
+    } else {
+        const size_t row = (size_t)bh * a.Nq + r0;
+        base = reinterpret_cast<char*>(a.O + row * a.d);
+        lse = a.LSE + row;
+        bytes = (size_t)(r1 - r0) * a.d * sizeof(half_t);
+    }
+    const u4 z = {0u, 0u, 0u, 0u};
+    const size_t whole = bytes / 16;
+    for (size_t i = tid; i < whole; i += nthreads) __builtin_nontemporal_store(z, reinterpret_cast<u4_anyalign*>(base + 16 * i));
+    if (tid == 0 && (bytes & 15) != 0) {
+        if (whole > 0) {
+            *reinterpret_cast<u4_anyalign*>(base + bytes - 16) = z;
+        } else {
+            for (size_t i = 0; i < bytes; i += 2) *reinterpret_cast<uint16_t*>(base + i) = 0;
+        }
+    }
+    for (int i = tid; i < r1 - r0; i += nthreads) lse[i] = -INFINITY;
+}
+
 // Position of a work-group in the launch's work order.  The order is "heaviest first", which balances a launch that
 // makes several rounds: whichever place frees up takes the heaviest work-group left.  But the work-groups of the first
 // round are not placed by load: the dispatcher deals work-group i to XCD i % 8 and there to CU (i / 8) % 32, so that with

@@ -120,6 +120,10 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     }
     const int tile_begin = kmin / BC;
     const int ntiles = kmax > kmin ? (kmax + BC - 1) / BC - tile_begin : 0;
+    if (!kStamp && ntiles == 0) {  // (the instrumented twins take the long way and report their stages)
+        store_empty_rows(a, bh, split, q0, q0 + C::BR < Nq ? q0 + C::BR : Nq, tid, 512);
+        return;
+    }
 
     // ---- this lane's query row and its interval of allowed keys
     // Row block of this wave: SIMD s hosts waves s and s + 4; giving them row blocks s and 7 - s evens out how long

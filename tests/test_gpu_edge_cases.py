@@ -99,6 +99,32 @@ def test_nq_differs_from_nk(fa, oracle, Nq, Nk):
         check_o_lse(o, lse, O, L, f"Nq={Nq} Nk={Nk} {list(kw)}")
 
 
+@pytest.mark.parametrize("d", [128, 72, 31, 9, 3])
+def test_row_blocks_without_visible_keys(fa, oracle, d):
+    """Nq > Nk under a causal mask: whole row blocks see no key and are filled with O = 0, LSE = -inf by work-groups that
+    request nothing (one contiguous piece of memory per block, at the alignment the head dim leaves it: 16-byte stores,
+    the last one ending with the piece; pieces shorter than 16 bytes element by element).  Unsplit in both tiled kernels,
+    and in three splits, where the empty work-groups fill their partial results."""
+    import torch
+    B, H, Nq, Nk = 1, 3, 700, 150
+    q, k, v = _qkv(B, H, Nq, Nk, d, seed=300 + d)
+    O, L = oracle_forward_batched(oracle, q, k, v, causal=True)
+    assert np.isneginf(L[..., :Nq - Nk]).all() and not np.isneginf(L[..., Nq - Nk:]).any()
+    for hint in ((fa.KERNEL_4WAVE, fa.KERNEL_8WAVE) if d == 128 else (0,)):
+        o = torch.full((B, H, Nq, d), float("nan"), dtype=torch.float16, device="cuda")
+        lse = torch.full((B, H, Nq), float("nan"), dtype=torch.float32, device="cuda")
+        fa.flash_forward_splitkv(q, k, v, num_splits=1, causal=True, out=o, lse=lse, kernel_hint=hint)
+        check_o_lse(o, lse, O, L, f"d={d} hint={hint}")
+        assert (o[..., :Nq - Nk, :] == 0).all()
+    o3, lse3, ws = fa.flash_forward_splitkv(q, k, v, num_splits=3, causal=True, return_partials=True)
+    check_o_lse(o3, lse3, O, L, f"d={d} three splits")
+    # a single row shorter than 16 bytes per head slice, nothing visible
+    q1, k1, v1 = _qkv(1, 2, 2, 1, d, seed=d)
+    o1, l1 = fa.flash_forward(q1, k1, v1, causal=True)
+    O1, L1 = oracle_forward_batched(oracle, q1, k1, v1, causal=True)
+    check_o_lse(o1, l1, O1, L1, f"d={d} two rows, one key")
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_many_head_slices_in_chunks(fa, oracle, causal):
     """With far more work-groups than the GPU holds at once the kernels deal the head slices out in chunks (here 256
