@@ -182,10 +182,37 @@ long long tiled_groups(const flash_params* p, const fa::FwdArgs& a)
 // The estimate for s splits: k (a + b t) / rho + [s > 1] (c0 + s * partials), t = tiles of a work-group (the heaviest one
 // plus k - 1 average ones), b = microseconds per 64-key tile of a work-group alone on its CU, rho the gain of k side by
 // side.  Over 21 swept shapes the count it picks is within 5 % of the best measured one on 19 (the others: 5.4 % and
-// 15 %); the reference's rule with 256 CUs: 12 of 21, the worst 6.8 times slower than the best count.  Costs the host
-// up to 0.2 ms on very long sequences (a loop over row blocks per candidate count): callers on a tight loop pass an
-// explicit count, or the one flash_splitkv_resolve_splits returned for the shape.
+// 15 %); the reference's rule with 256 CUs: 12 of 21, the worst 6.8 times slower than the best count.
+int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode);
+
+// The estimate walks the row blocks once per candidate count (up to 0.26 ms on a causal sequence of 65536 rows), and
+// callers in a loop ask for the same few shapes again and again: each thread remembers the answers to its last four
+// distinct requests.  Everything the estimate reads is part of the key.
 int auto_splits_tiled(const flash_params* p, int n_blocks, bool decode = false)
+{
+    struct Key {
+        int B, H, H_kv, Nq, Nk, d, causal, wl, wr, hint, flags;
+        bool operator==(const Key& o) const
+        {
+            return B == o.B && H == o.H && H_kv == o.H_kv && Nq == o.Nq && Nk == o.Nk && d == o.d && causal == o.causal &&
+                   wl == o.wl && wr == o.wr && hint == o.hint && flags == o.flags;
+        }
+    };
+    struct Entry { Key key; int splits; bool valid; };
+    static thread_local Entry memo[4];
+    static thread_local int next = 0;
+    const Key key = {p->B, p->H, p->H_kv, p->Nq, p->Nk, p->d, p->is_causal, window_left_of(p), window_right_of(p), p->kernel_hint,
+                     tiled_variant(p) | (p->softmax_scale > 0.0f ? 8 : 0) | (p->scores_out ? 16 : 0) | (decode ? 32 : 0) |
+                         (p->dropout_p > 0.0f && flash_dropout_threshold(p->dropout_p) == 0 ? 64 : 0)};
+    for (const Entry& e : memo)
+        if (e.valid && e.key == key) return e.splits;
+    const int splits = auto_splits_tiled_uncached(p, n_blocks, decode);
+    memo[next] = Entry{key, splits, true};
+    next = (next + 1) % 4;
+    return splits;
+}
+
+int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode)
 {
     const int wl = window_left_of(p), wr = window_right_of(p);
     const bool vec = (tiled_variant(p) & 1) != 0;

@@ -203,6 +203,34 @@ def test_automatic_split_count_stays_in_range_on_random_shapes(fa):
         assert (ob, lb) == (rows * d * 4, rows * 4)
 
 
+def test_automatic_split_count_is_remembered_per_request(fa):
+    """The library remembers the answers of a thread's last four distinct automatic requests.  Ten requests that differ
+    in one field each (shape, mask, window, K/V heads, kernel hint), asked in turn three times over -- so that every one
+    is evicted before it comes round again -- and twice in a row: always the first answer."""
+    import threading
+    base = dict(B=1, H=8, Nq=4096, Nk=4096, d=128, causal=True, window=(-1, -1), H_kv=8, kernel_hint=0)
+    variants = [dict(), dict(B=2), dict(H=4, H_kv=4), dict(Nq=2048), dict(Nk=16384), dict(d=64), dict(causal=False),
+                dict(window=(1024, -1)), dict(H_kv=2), dict(kernel_hint=fa.KERNEL_4WAVE)]
+
+    def ask(v):
+        c = dict(base, **v)
+        return fa.resolve_splits(c["B"], c["H"], c["Nq"], c["Nk"], c["d"], 0, causal=c["causal"], window=c["window"],
+                                 H_kv=c["H_kv"], kernel_hint=c["kernel_hint"])
+
+    first = [ask(v) for v in variants]
+    assert len(set(first)) > 1, "the variants should not all resolve to the same count"
+    for _ in range(3):
+        assert [ask(v) for v in variants] == first
+    for v, want in zip(variants, first):
+        assert ask(v) == want and ask(v) == want
+    # another thread has a memory of its own
+    got = []
+    t = threading.Thread(target=lambda: got.extend(ask(v) for v in variants))
+    t.start()
+    t.join()
+    assert got == first
+
+
 def test_stage_stamp_buffer_size(fa):
     L = fa.lib()
     nb = C.c_size_t(99)
