@@ -16,6 +16,9 @@ typedef float v2f __attribute__((ext_vector_type(2)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+// 16 bytes at any 2-byte / 4-byte boundary (the hardware runs in unaligned access mode): rows of d % 8 != 0 elements
+typedef v4u __attribute__((aligned(2))) v4u_anyalign;
+typedef v4f __attribute__((aligned(4))) v4f_anyalign;
 // operand type of the ds_read_b64_tr_b16 builtin
 typedef __fp16 v4hp __attribute__((__vector_size__(4 * sizeof(__fp16))));
 
@@ -62,6 +65,19 @@ struct FwdArgs {
 
 __device__ __forceinline__ int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
+// Q chunk for the chunk position at column col (a multiple of 8) of a row of d >= 8 elements at any alignment, where the
+// position behind the row's whole chunks stands for columns d - 8 ... d - 1 and v holds what was loaded from there (see
+// fwd_kernel.h): the columns that the chunk before has covered already are zeroed, and so are positions past the row.
+__device__ __forceinline__ v8h mask_q_chunk_anyalign(v4u v, int col, int d)
+{
+    union { v4u u; v8h h; } t;
+    t.u = v;
+    const int covered = col + 8 <= d ? 0 : col < d ? 8 - (d & 7) : 8;  // leading elements that must not count
+#pragma unroll
+    for (int e = 0; e < 8; ++e) t.h[e] = e >= covered ? t.h[e] : (half_t)0.0f;
+    return t.h;
+}
+
 // A work-group whose rows see no key at all (rows above a causal diagonal that starts below them, a split of the key
 // range beyond their mask): O = 0 and LSE = -inf for rows [r0, r1) of head slice bh, or the same in the slice's partial
 // results of split `split`.  The rows are one contiguous piece of memory; it is filled with 16-byte stores at whatever
@@ -69,8 +85,6 @@ __device__ __forceinline__ int wave_uniform(int v) { return __builtin_amdgcn_rea
 // is requested: such a group is done in the time of its stores.
 __device__ __forceinline__ void store_empty_rows(const FwdArgs& a, int bh, int split, int r0, int r1, int tid, int nthreads)
 {
-    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
-    typedef u4 __attribute__((aligned(2))) u4_anyalign;
     char* base;
     float* lse;
     size_t bytes;
@@ -85,12 +99,12 @@ __device__ __forceinline__ void store_empty_rows(const FwdArgs& a, int bh, int s
         lse = a.LSE + row;
         bytes = (size_t)(r1 - r0) * a.d * sizeof(half_t);
     }
-    const u4 z = {0u, 0u, 0u, 0u};
+    const v4u z = {0u, 0u, 0u, 0u};
     const size_t whole = bytes / 16;
-    for (size_t i = tid; i < whole; i += nthreads) __builtin_nontemporal_store(z, reinterpret_cast<u4_anyalign*>(base + 16 * i));
+    for (size_t i = tid; i < whole; i += nthreads) __builtin_nontemporal_store(z, reinterpret_cast<v4u_anyalign*>(base + 16 * i));
     if (tid == 0 && (bytes & 15) != 0) {
         if (whole > 0) {
-            *reinterpret_cast<u4_anyalign*>(base + bytes - 16) = z;
+            *reinterpret_cast<v4u_anyalign*>(base + bytes - 16) = z;
         } else {
             for (size_t i = 0; i < bytes; i += 2) *reinterpret_cast<uint16_t*>(base + i) = 0;
         }

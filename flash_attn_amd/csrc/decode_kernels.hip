@@ -54,17 +54,17 @@ __global__ void __launch_bounds__(256) decode_split_kernel(const FwdArgs a)
     const int bh0 = (blockIdx.x % BHG) * G;  // first of the G query slices of this work-group
     const int split = blockIdx.x / BHG;
     const int d = a.d, Nk = a.Nk;
+    // Rows of any length from eight elements on, at any 2-byte alignment: a lane behind the row's whole chunks works
+    // on the row's last 16 bytes, columns d - 8 ... d - 1 (no load leaves the row), with q zeroed where the lane before
+    // has covered a column already; lanes past the row do the same with q = 0.
     const int col = 8 * c;
-    const bool cvalid = col < d;
-    const int colc = cvalid ? col : d - 8;
+    const int colc = col + 8 <= d ? col : d - 8;
 
     union U8 { v4u u; v8h h; v2h p[4]; };
     U8 qv[G];
 #pragma unroll
-    for (int gq = 0; gq < G; ++gq) {
-        qv[gq].u = *reinterpret_cast<const v4u*>(a.Q + (size_t)(bh0 + gq) * d + colc);
-        if (!cvalid) qv[gq].u = v4u{0u, 0u, 0u, 0u};
-    }
+    for (int gq = 0; gq < G; ++gq)
+        qv[gq].h = mask_q_chunk_anyalign(*reinterpret_cast<const v4u_anyalign*>(a.Q + (size_t)(bh0 + gq) * d + colc), col, d);
 
     // the single query row sits at position ii = Nk - 1 (row index i + Nk - Nq): causal / right window never cut
     const int ii = Nk - 1;
@@ -105,13 +105,13 @@ __global__ void __launch_bounds__(256) decode_split_kernel(const FwdArgs a)
             const int j = kb + i * KPI + kg;
             const size_t off = (size_t)(j < kend ? j : kend - 1) * d;
             // (non-temporal: K and V are read once; as ordinary loads they measured 5.9 instead of 6.8 TB/s)
-            kr[i].u = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(Kbh + off));
+            kr[i].u = __builtin_nontemporal_load(reinterpret_cast<const v4u_anyalign*>(Kbh + off));
         }
 #pragma unroll
         for (int i = 0; i < U; ++i) {
             const int j = kb + i * KPI + kg;
             const size_t off = (size_t)(j < kend ? j : kend - 1) * d;
-            vr[i].u = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(Vbh + off));
+            vr[i].u = __builtin_nontemporal_load(reinterpret_cast<const v4u_anyalign*>(Vbh + off));
         }
     };
     auto consume = [&](int kb, const U8 (&kr)[U], const U8 (&vr)[U]) __attribute__((always_inline)) {
@@ -194,12 +194,17 @@ __global__ void __launch_bounds__(256) decode_split_kernel(const FwdArgs a)
             }
             const float inv = L > 0.0f ? 1.0f / L : 0.0f;
             const float lse = L > 0.0f ? __builtin_fmaf(M, kLn2, fast_log2(L) * kLn2) : -INFINITY;
+            // column of position tid: the eight positions behind the row's whole chunks hold columns d - 8 ... d - 1, of
+            // which the first 8 - d % 8 were written by the positions before
+            const int c0 = d & ~7, rem = d & 7;
+            const int tcol = tid < c0 ? tid : tid - (8 - rem);
+            const bool ok = tid < c0 || (rem != 0 && tid < c0 + 8 && tcol >= c0);
             if (a.num_splits > 1) {
                 const size_t prow = (size_t)bh * a.num_splits + split;  // Nq == 1
-                if (tid < d) a.O_partial[prow * d + tid] = o * inv;
+                if (ok) a.O_partial[prow * d + tcol] = o * inv;
                 if (tid == 0) a.LSE_partial[prow] = lse;
             } else {
-                if (tid < d) a.O[(size_t)bh * d + tid] = (half_t)(o * inv);
+                if (ok) a.O[(size_t)bh * d + tcol] = (half_t)(o * inv);
                 if (tid == 0) a.LSE[bh] = lse;
             }
         }

@@ -301,7 +301,7 @@ int resolve_splits(const flash_params* p)
         const int hk = p->H_kv > 0 ? p->H_kv : p->H;
         const int G = p->H / (hk > 0 ? hk : 1);
         const bool heads_as_rows = G >= 4 && !p->alibi_slopes && window_left_of(p) < 0 && p->dropout_p == 0.0f;
-        const bool one_row_kernel = !heads_as_rows && p->d % 8 == 0 && p->dropout_p == 0.0f && p->softmax_scale > 0.0f;
+        const bool one_row_kernel = !heads_as_rows && p->d >= 8 && p->dropout_p == 0.0f && p->softmax_scale > 0.0f;
         if (one_row_kernel) {
             // Each wave keeps the 2 U loads of its next key block in flight while it works on the current one (64-128 KiB
             // per work-group), so one work-group per CU already covers the memory latency.  Measured over 61 random
@@ -322,7 +322,7 @@ int resolve_splits(const flash_params* p)
             s = (int)(want < n_blocks ? want : n_blocks);
         } else {
             // The tiled kernel serves four or more query heads of a K/V head together (heads as the rows of one problem per
-            // K/V head) and every request the one-row kernel cannot (d % 8 != 0, dropout): the estimate of the tiled path
+            // K/V head) and every request the one-row kernel cannot (d < 8, dropout): the estimate of the tiled path
             // for that problem.
             flash_params r = *p;
             if (heads_as_rows) {
@@ -392,8 +392,8 @@ int splitkv_route(const flash_params* p, fa::FwdArgs* a)
         a->Tr = (a->Nq + kRowsPerGroup - 1) / kRowsPerGroup;
         return kRouteTiled;
     }
-    // one query row per head, 16-byte rows, no dropout: bandwidth-bound streaming kernel
-    if (p->Nq == 1 && p->d % 8 == 0 && p->dropout_p == 0.0f && p->softmax_scale > 0.0f) return kRouteStream;
+    // one query row per head, rows of eight elements or more, no dropout: bandwidth-bound streaming kernel
+    if (p->Nq == 1 && p->d >= 8 && p->dropout_p == 0.0f && p->softmax_scale > 0.0f) return kRouteStream;
     return kRouteTiled;
 }
 

@@ -111,20 +111,9 @@ __device__ __forceinline__ v4u load_chunk_unpadded(const half_t* __restrict__ ro
 //       bytes; chunks past the row yield columns that are never stored.
 // Element by element, a 64 x 32 tile took 16 two-byte loads per thread with an address computation each, where this takes
 // two loads and no arithmetic on the data.
-typedef v4u __attribute__((aligned(2))) v4u_anyalign;
-typedef v4f __attribute__((aligned(4))) v4f_anyalign;
 __device__ __forceinline__ v4u load_chunk_anyalign(const half_t* __restrict__ rowp, int col, int d)
 {
     return *reinterpret_cast<const v4u_anyalign*>(rowp + (col + 8 <= d ? col : d - 8));
-}
-__device__ __forceinline__ v8h mask_q_chunk_anyalign(v4u v, int col, int d)
-{
-    union { v4u u; v8h h; } t;
-    t.u = v;
-    const int covered = col + 8 <= d ? 0 : col < d ? 8 - (d & 7) : 8;  // leading elements that must not count
-#pragma unroll
-    for (int e = 0; e < 8; ++e) t.h[e] = e >= covered ? t.h[e] : (half_t)0.0f;
-    return t.h;
 }
 
 // Running maximum is only raised when some row of the wave outgrows it by more than this many powers of two;

@@ -331,11 +331,28 @@ def test_splitkv_heuristic_and_decode_variants(fa, oracle):
             o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=S, **kw)
             O, L = oracle_forward_batched(oracle, q, k, v, **okw)
             check_o_lse(o, lse, O, L, f"decode d={d} Nk={Nk} S={S} {list(kw)}")
-    # Nq == 1 with an odd head dim or dropout falls back to the tiled kernel
-    q, k, v = _qkv(1, 2, 1, 900, 31, seed=9)
+    # Nq == 1 with rows shorter than a chunk falls back to the tiled kernel
+    q, k, v = _qkv(1, 2, 1, 900, 5, seed=9)
     o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=4)
     O, L = oracle_forward_batched(oracle, q, k, v)
-    check_o_lse(o, lse, O, L, "decode odd d")
+    check_o_lse(o, lse, O, L, "decode d < 8")
+
+
+# The decode kernel on rows at any alignment: every length of the partial last chunk in every bucket of its lane mapping
+# (4, 8 or 16 lanes per key), plain / window + ALiBi, two query heads per K/V head, unsplit and split (where the partial
+# rows take the same column mapping); d = 8 ... 15 are rows of a single, partial or whole, chunk.
+@pytest.mark.parametrize("d", [8, 9, 11, 14, 15, 17, 23, 26, 31, 33, 37, 44, 50, 63, 65, 71, 78, 92, 100, 109, 121, 127])
+def test_decode_rows_at_any_alignment(fa, oracle, d):
+    B, H, Hk, Nk = 2, 4, 2, 700 + d
+    q = randn_f16_gpu((B, H, 1, d), 7000 + d)
+    k, v = randn_f16_gpu((B, Hk, Nk, d), 7100 + d), randn_f16_gpu((B, Hk, Nk, d), 7200 + d)
+    sl, sl_t = _slopes(oracle, H)
+    kr, vr = k.repeat_interleave(H // Hk, dim=1), v.repeat_interleave(H // Hk, dim=1)
+    for kw, okw in ((dict(), dict()), (dict(window=(300, 0), alibi_slopes=sl_t), dict(window=(300, 0), slopes=sl))):
+        O, L = oracle_forward_batched(oracle, q, kr, vr, **okw)
+        for S in (1, 3):
+            o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=S, **kw)
+            check_o_lse(o, lse, O, L, f"decode d={d} S={S} {sorted(kw)}")
 
 
 # grouped-query / multi-query attention: K, V carry H_kv heads and query head h reads K/V head h // (H // H_kv); the
