@@ -134,6 +134,13 @@ void fill_args(const flash_params* p, int splits, fa::FwdArgs* a)
 }
 
 // variant bits of the tiled kernel for p (kVarVec | kVarAlibi | kVarDropout of fwd_kernel.h)
+// requests that only the tiled kernel's instance which serves every request takes (fa::fwd_needs_every_instance)
+bool needs_every_instance(const flash_params* p)
+{
+    return p->softmax_scale <= 0.0f || p->scores_out || p->d < 8 ||
+           (p->dropout_p > 0.0f && flash_dropout_threshold(p->dropout_p) == 0);
+}
+
 int tiled_variant(const flash_params* p)
 {
     // A non-positive scale does not commute with the row maximum: only the any-alignment instance that serves every request scales first.
@@ -160,7 +167,7 @@ int launch_tiled(const flash_params* p, const fa::FwdArgs& a, hipStream_t st)
 // work-groups of the tiled launch for the (final) arguments a
 long long tiled_groups(const flash_params* p, const fa::FwdArgs& a)
 {
-    const bool pp = a.d > 96 && fa::fwd_uses_pingpong(a.d, (tiled_variant(p) & 1) != 0, a.Nq, a.causal, a.wl, a.wr,
+    const bool pp = a.d > 96 && fa::fwd_uses_pingpong(a.d, !needs_every_instance(p), a.Nq, a.causal, a.wl, a.wr,
                                                       (long long)a.B * a.H * a.num_splits, a.kernel_hint);
     const int rows = pp ? 256 : kRowsPerGroup;
     return (long long)((a.Nq + rows - 1) / rows) * a.B * a.H * a.num_splits;
@@ -215,8 +222,8 @@ int auto_splits_tiled(const flash_params* p, int n_blocks, bool decode = false)
 int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode)
 {
     const int wl = window_left_of(p), wr = window_right_of(p);
-    const bool vec = (tiled_variant(p) & 1) != 0;
-    const bool pp = fa::fwd_uses_pingpong(p->d, vec, p->Nq, p->is_causal, wl, wr, (long long)p->B * p->H, p->kernel_hint);
+    const bool every = needs_every_instance(p);
+    const bool pp = fa::fwd_uses_pingpong(p->d, !every, p->Nq, p->is_causal, wl, wr, (long long)p->B * p->H, p->kernel_hint);
     const int rows = pp ? 256 : kRowsPerGroup;
     const int Tr = (p->Nq + rows - 1) / rows;
     const long long slices = (long long)p->B * p->H;
@@ -227,8 +234,6 @@ int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode)
     // 1.0-1.2 x the bucket-wide instance), x 1.5 for the instance that serves every request (tiles staged through
     // registers)
     static const float kTile[5] = {0.0f, 0.5f, 0.72f, 0.88f, 1.0f};
-    const bool every = p->softmax_scale <= 0.0f || p->scores_out || p->d < 8 ||
-                       (p->dropout_p > 0.0f && flash_dropout_threshold(p->dropout_p) == 0);
     const bool dma = !every && p->d == 32 * bucket;
     // (decode launches, whose tiles no other work-group has asked for before: twice that, and 0.04 us per split for
     // the combine of their few rows; fitted to 55 random decode shapes of the tiled routes)

@@ -1,9 +1,9 @@
 // Instances of the tiled forward kernels for the head-dim bucket d <= 128.
 #include "fwd_pp_kernel.h"
 namespace fa {
-bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr, long long slices, int hint)
+bool fwd_uses_pingpong(int d, bool direct, int Nq, int causal, int wl, int wr, long long slices, int hint)
 {
-    // d == 128, more than one 128-row block of queries and no narrow window: the 8-wave ping-pong kernel (measured
+    // 96 < d <= 128, more than one 128-row block of queries and no narrow window: the 8-wave ping-pong kernel (measured
     // 3-18 % faster than the 4-wave kernel there; slower for d = 64 and for windows much smaller than its 256-row
     // block, which make it compute mostly masked tiles).  Short causal problems stay with the 4-wave kernel: up to
     // 1024 rows the diagonal, where the waves of a 256-row block run out of keys one after the other, is too large a
@@ -13,8 +13,9 @@ bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr, long
     // where an unmasked launch is one round that fills three quarters of the CUs or more (192 ... 256 work-groups:
     // measured 3-13 % faster with the 8-wave kernel on eleven random shapes of twelve, 128 and fewer 15-35 % slower).
     // The caller's hint (flash_params::kernel_hint: 1 = 4-wave, 2 = 8-wave) overrides these preferences for A/B runs
-    // and tests; the 8-wave kernel still needs d == 128 in whole 16-byte rows and more than 128 query rows.
-    const bool able = vec && d == 128 && Nq > 128;
+    // and tests; the 8-wave kernel still needs 96 < d <= 128, more than 128 query rows and a request that the instances
+    // with tiles straight into LDS serve (direct: not one for the instance that serves every request).
+    const bool able = direct && d > 96 && d <= 128 && Nq > 128;
     if (hint == 1) return false;
     if (hint == 2) return able;
     const bool narrow_window = (wl >= 0 && wl < 512) || (wr >= 0 && wr < 512 && !causal);
@@ -27,7 +28,7 @@ bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr, long
 int launch_fwd_d128(const FwdArgs& a, int variant, int nb, hipStream_t st)
 {
     (void)nb;
-    if (fwd_uses_pingpong(a.d, (variant & kVarVec) != 0, a.Nq, a.causal, a.wl, a.wr, (long long)a.B * a.H * a.num_splits,
+    if (fwd_uses_pingpong(a.d, !fwd_needs_every_instance(a, variant), a.Nq, a.causal, a.wl, a.wr, (long long)a.B * a.H * a.num_splits,
                           a.kernel_hint))
         return launch_fwd_pp_bucket<128>(a, variant, st);
     return launch_fwd_bucket<128, 1>(a, variant, st);

@@ -908,7 +908,7 @@ int launch_fwd_d96(const FwdArgs& a, int variant, int nb, hipStream_t st);
 int launch_fwd_d128(const FwdArgs& a, int variant, int nb, hipStream_t st);
 // whether launch_fwd_d128 takes the 8-wave kernel (256 query rows per work-group instead of 128)
 // (slices = B * H * num_splits; hint = flash_params::kernel_hint)
-bool fwd_uses_pingpong(int d, bool vec, int Nq, int causal, int wl, int wr, long long slices, int hint);
+bool fwd_uses_pingpong(int d, bool direct, int Nq, int causal, int wl, int wr, long long slices, int hint);
 
 // Head slices per chunk of the work-group order: the smallest divisor of the slice count (a multiple of 8, which keeps a
 // slice on one XCD) whose chunk still holds twice the work-groups that run at once -- enough for "heaviest row blocks
@@ -961,6 +961,12 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
 // The instances of a bucket: {d == bucket, d % 8 == 0} x {plain, ALiBi, ALiBi with every visible key at or left of its
 // row, dropout, both}, for rows at any alignment (d % 8 != 0) {plain, ALiBi, dropout, both}, and the one that serves
 // every other request.  ST = kVarStamp selects their instrumented twins (debug time stamps).
+// requests that only the instance which serves every request takes (kEvery in fwd_kernel)
+inline bool fwd_needs_every_instance(const FwdArgs& a, int variant)
+{
+    return a.scale_log2 <= 0.0f || a.scores_out != nullptr || a.d < 8 || ((variant & kVarDropout) && a.drop_thr == 0);
+}
+
 template <int D, int NB, int ST>
 inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
 {
@@ -972,8 +978,7 @@ inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
         // threshold 0 make them identities) for every other request: a non-positive scale (its ALiBi step is where the
         // scores are scaled ahead of the row maximum), the score dump, rows of fewer than eight elements, a dropout
         // threshold of 0
-        const bool every = a.scale_log2 <= 0.0f || a.scores_out != nullptr || a.d < 8 || ((feat & kVarDropout) && a.drop_thr == 0);
-        if (every) e = launch_fwd_instance<D, NB, ST | kVarAlibi | kVarDropout | kVarEvery>(a, st);
+        if (fwd_needs_every_instance(a, variant)) e = launch_fwd_instance<D, NB, ST | kVarAlibi | kVarDropout | kVarEvery>(a, st);
         else if (feat == 0) e = launch_fwd_instance<D, NB, ST>(a, st);
         else if (feat == kVarAlibi) e = launch_fwd_instance<D, NB, ST | kVarAlibi>(a, st);
         else if (feat == kVarDropout) e = launch_fwd_instance<D, NB, ST | kVarDropout>(a, st);

@@ -1,4 +1,5 @@
-// Ping-pong variant of the tiled forward kernel for head dim 128 (d == D == 128).
+// Ping-pong variant of the tiled forward kernel for the head-dim bucket 128 (96 < d <= 128; rows shorter than 128 elements
+// and rows at any 2-byte alignment as in fwd_kernel.h: chunk positions behind a row's whole chunks hold its last 16 bytes).
 //
 // Same math as fwd_kernel.h (S^T = K Q^T and O^T += V^T P^T on MFMA 32x32x16, Q in registers, online softmax per
 // lane, 64-key tiles).  What changes is the schedule and the way tiles reach LDS:
@@ -69,7 +70,8 @@ __device__ __forceinline__ void lds_barrier_keep(void)
 template <int D, int VAR>
 __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
 {
-    constexpr bool kAlibi = (VAR & kVarAlibi) != 0, kDropout = (VAR & kVarDropout) != 0, kStamp = (VAR & kVarStamp) != 0;
+    constexpr bool kAlibi = (VAR & kVarAlibi) != 0, kDropout = (VAR & kVarDropout) != 0, kStamp = (VAR & kVarStamp) != 0,
+                   kFullD = (VAR & kVarFullD) != 0;
     using C = PPCfg<D>;
     Stamps<kStamp> stamps;
     stamps.take(0);
@@ -101,7 +103,9 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
     const int m_block = a.Tr - 1 - mi;
     const int h = bh % a.H;
     const int Nq = a.Nq, Nk = a.Nk;
-    constexpr int d = D;
+    const int d = kFullD ? D : a.d;  // 8 <= d <= D
+    // byte offset of chunk position c inside a row of global memory
+    auto chunk_offset = [&](int c) { return kFullD ? c * 16 : (c * 8 + 8 <= d ? c * 16 : (d - 8) * 2); };
     const int shift = Nk - Nq;
     const int q0 = m_block * C::BR;
 
@@ -191,8 +195,8 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         const int sigma = 2 * (dkey & 3) + ((dkey >> 2) & 1);
         // (unsigned: a slice may be just short of 4 GiB)
         const uint32_t row0 = (uint32_t)(tile_begin * BC + dkey) * (uint32_t)(d * 2);
-        kgo = row0 + (uint32_t)((slot ^ (dkey & 15)) << 4);
-        vgo = row0 + (uint32_t)((((slot >> 1) ^ sigma) << 5) | ((slot & 1) << 4));
+        kgo = row0 + (uint32_t)chunk_offset(slot ^ (dkey & 15));
+        vgo = row0 + (uint32_t)chunk_offset((((slot >> 1) ^ sigma) << 1) | (slot & 1));
     }
     const char* const Kb = reinterpret_cast<const char*>(Kbh);
     const char* const Vb = reinterpret_cast<const char*>(Vbh);
@@ -514,7 +518,7 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         for (int x = 0; x < 8; ++x) {
             const int rl = 4 * x + (lane >> 4);  // row of the wave's 32
             const int gi = q0 + rblk * 32 + rl;
-            const uint32_t off = (uint32_t)(gi < Nq ? gi : Nq - 1) * (uint32_t)(d * 2) + (uint32_t)(((lane & 15) ^ (rl & 15)) << 4);
+            const uint32_t off = (uint32_t)(gi < Nq ? gi : Nq - 1) * (uint32_t)(d * 2) + (uint32_t)chunk_offset((lane & 15) ^ (rl & 15));
             dma_kib(Qb, off, qst + x * 1024);
         }
         if (ntiles > 0) {
@@ -536,6 +540,14 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
         for (int ks = 0; ks < KS; ++ks)
             qf[ks] = *reinterpret_cast<FA_LDS const v8h*>(
                 reinterpret_cast<FA_LDS const char*>(static_cast<uintptr_t>(qbase ^ (uint32_t)(ks << 5))));
+        if constexpr (!kFullD) {  // zeroes where the chunk before has covered a column already, and past the row
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                union { v8h h; v4u u; } t;
+                t.h = qf[ks];
+                qf[ks] = mask_q_chunk_anyalign(t.u, 16 * ks + 8 * g, d);
+            }
+        }
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));  // Q is in registers before the loop
@@ -603,7 +615,14 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
                         const int dc = 32 * mb + 8 * rg + 4 * g;
                         v4f o = {oacc[mb][4 * rg] * inv, oacc[mb][4 * rg + 1] * inv, oacc[mb][4 * rg + 2] * inv,
                                  oacc[mb][4 * rg + 3] * inv};
-                        *reinterpret_cast<v4f*>(op + dc) = o;
+                        if constexpr (kFullD) {
+                            *reinterpret_cast<v4f*>(op + dc) = o;
+                        } else {
+                            // the chunk position behind the row's whole chunks holds columns d - 8 ... d - 1
+                            const int c0 = d & ~7, rem = d & 7;
+                            if (dc < c0 || (rem != 0 && dc < c0 + 8))
+                                *reinterpret_cast<v4f_anyalign*>(op + (dc < c0 ? dc : dc - (8 - rem))) = o;
+                        }
                     }
             }
         } else {
@@ -629,8 +648,13 @@ __global__ void __launch_bounds__(512, 2) fwd_pp_kernel(const FwdArgs a)
                 const int rl = 4 * x + (lane >> 4);
                 const int gi = q0 + rblk * 32 + rl;
                 const v4u val = *reinterpret_cast<FA_LDS const v4u*>(ost + x * 1024 + lane * 16);
-                if (gi < Nq)
-                    __builtin_nontemporal_store(val, reinterpret_cast<v4u*>(Ob + (size_t)gi * d * 2 + (((lane & 15) ^ (rl & 15)) << 4)));
+                const int c = (lane & 15) ^ (rl & 15);
+                if constexpr (kFullD) {
+                    if (gi < Nq) __builtin_nontemporal_store(val, reinterpret_cast<v4u*>(Ob + (size_t)gi * d * 2 + (c << 4)));
+                } else {
+                    if (gi < Nq && c * 8 < d)
+                        __builtin_nontemporal_store(val, reinterpret_cast<v4u_anyalign*>(Ob + (size_t)gi * d * 2 + chunk_offset(c)));
+                }
             }
         }
     }
@@ -657,16 +681,24 @@ inline hipError_t launch_fwd_pp_instance(const FwdArgs& a, hipStream_t st)
     return launch_kernel(kern, dim3((unsigned)groups), dim3(512), C::SMEM, st, b);
 }
 
-// d == D, 16-byte rows: {plain, ALiBi, dropout, both}; ST = kVarStamp: their instrumented twins
+// {d == D, shorter rows} x {plain, ALiBi, dropout, both}; ST = kVarStamp: their instrumented twins
 template <int D, int ST>
 inline int launch_fwd_pp_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
 {
     const int feat = variant & (kVarAlibi | kVarDropout);
     hipError_t e;
-    if (feat == 0) e = launch_fwd_pp_instance<D, ST>(a, st);
-    else if (feat == kVarAlibi) e = launch_fwd_pp_instance<D, ST | kVarAlibi>(a, st);
-    else if (feat == kVarDropout) e = launch_fwd_pp_instance<D, ST | kVarDropout>(a, st);
-    else e = launch_fwd_pp_instance<D, ST | kVarAlibi | kVarDropout>(a, st);
+    if (a.d == D) {
+        constexpr int V = ST | kVarFullD;
+        if (feat == 0) e = launch_fwd_pp_instance<D, V>(a, st);
+        else if (feat == kVarAlibi) e = launch_fwd_pp_instance<D, V | kVarAlibi>(a, st);
+        else if (feat == kVarDropout) e = launch_fwd_pp_instance<D, V | kVarDropout>(a, st);
+        else e = launch_fwd_pp_instance<D, V | kVarAlibi | kVarDropout>(a, st);
+    } else {
+        if (feat == 0) e = launch_fwd_pp_instance<D, ST>(a, st);
+        else if (feat == kVarAlibi) e = launch_fwd_pp_instance<D, ST | kVarAlibi>(a, st);
+        else if (feat == kVarDropout) e = launch_fwd_pp_instance<D, ST | kVarDropout>(a, st);
+        else e = launch_fwd_pp_instance<D, ST | kVarAlibi | kVarDropout>(a, st);
+    }
     return (int)e;
 }
 

@@ -73,6 +73,34 @@ def test_any_alignment_instances(fa, oracle, d):
         check_o_lse(o3, lse3, O, L, f"d={d} {feat} three splits")
 
 
+# The 8-wave kernel on rows shorter than its 128-element bucket, in whole chunks (104, 112, 120) and at any alignment
+# (every length of the partial last chunk): plain, causal + ALiBi, window + dropout with the keep decisions dumped, ragged
+# Nq and Nk, unsplit and in three splits (fp32 partial rows with the same column mapping).
+@pytest.mark.parametrize("d", [97, 98, 99, 100, 101, 102, 103, 104, 110, 112, 119, 120, 127])
+def test_8wave_kernel_on_shorter_rows(fa, oracle, d):
+    import torch
+    B, H, Nq, Nk = 1, 2, 333, 471
+    q, k, v = _qkv(B, H, Nq, Nk, d, seed=3000 + d)
+    sl, sl_t = _slopes(oracle, H)
+    keep = oracle.dropout_keep_mask(11, d, 0.25, B, H, Nq, Nk)
+    cases = ((dict(), dict(), False),
+             (dict(causal=True, alibi_slopes=sl_t), dict(causal=True, slopes=sl), False),
+             (dict(window=(200, 50), dropout_p=0.25, seed=11, offset=d),
+              dict(window=(200, 50), keep_mask=torch.from_numpy(keep), p_drop=0.25), True))
+    for kw, okw, drop in cases:
+        O, L = oracle_forward_batched(oracle, q, k, v, **okw)
+        for S in (1, 3):
+            o, lse = fa.flash_forward_splitkv(q, k, v, num_splits=S, kernel_hint=fa.KERNEL_8WAVE, **kw)
+            check_o_lse(o, lse, O, L, f"8-wave d={d} S={S} {sorted(kw)}")
+            o4, lse4 = fa.flash_forward_splitkv(q, k, v, num_splits=S, kernel_hint=fa.KERNEL_4WAVE, **kw)
+            check_o_lse(o4, lse4, O, L, f"4-wave d={d} S={S} {sorted(kw)}")
+        if drop:
+            _, _, km = fa.flash_forward(q, k, v, return_keep_mask=True, kernel_hint=fa.KERNEL_8WAVE, **kw)
+            i, j = np.arange(Nq)[:, None] + (Nk - Nq), np.arange(Nk)[None, :]
+            vis = (j >= i - 200) & (j <= i + 50)
+            assert np.array_equal(km.cpu().numpy()[..., vis], keep[..., vis]), f"d={d}"
+
+
 # sequence lengths around the tile sizes (64-key tiles, 128-row groups); 1021 is the reference's checked-in seq_len
 @pytest.mark.parametrize("N", [1, 2, 31, 63, 64, 65, 127, 128, 129, 191, 257, 1000, 1021])
 def test_ragged_lengths(fa, oracle, N):
