@@ -83,23 +83,6 @@ __device__ __forceinline__ v4u load_chunk(const half_t* __restrict__ rowp, int c
     }
 }
 
-// The same for a chunk of a K or V tile, without the zeroes: columns >= d come back as copies of the row's last
-// elements.  For K they meet the zero columns of Q, for V they only reach rows of O^T that are never stored, so the
-// values do not matter as long as they are the row's own finite data -- and without the select the tile's loads are
-// not waited for until their data is written to LDS, behind the arithmetic of the current tile (with it, the compiler
-// placed the selects, and with them the wait for the whole tile, right behind the loads).
-template <bool kVec, bool kFullD>
-__device__ __forceinline__ v4u load_chunk_unpadded(const half_t* __restrict__ rowp, int col, int d)
-{
-    if constexpr (kFullD) {
-        return *reinterpret_cast<const v4u*>(rowp + col);
-    } else if constexpr (kVec) {
-        return *reinterpret_cast<const v4u*>(rowp + (col < d ? col : d - 8));
-    } else {
-        return load_chunk<kVec, kFullD>(rowp, col, d);
-    }
-}
-
 // Rows that start at any 2-byte boundary (d % 8 != 0), d >= 8: a chunk is still one 16-byte load -- the hardware runs in
 // unaligned access mode -- taken at the chunk's own column, or, for the row's last, partial chunk and for chunks past the
 // row, at column d - 8, so that no load ever leaves the row.  Nothing is moved into place afterwards: the last chunk
@@ -298,7 +281,11 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
         }
     }
 
-    // ---- tile staging: thread handles chunk ids tid + 256*x  ->  (row, chunk) of the 64 x CH tile
+    // ---- tile staging through registers (the instance that serves every request; all others request their tiles
+    // straight into LDS, below): thread handles chunk ids tid + 256*x  ->  (row, chunk) of the 64 x CH tile.  The
+    // loads of tile t+1 are issued in front of the arithmetic of tile t and waited for where their data is written to
+    // LDS behind it: nothing is computed on what was loaded (a select on it would drag the wait for the whole tile in
+    // front of the arithmetic).
     int ld_row[NLD], ld_col[NLD];
 #pragma unroll
     for (int x = 0; x < NLD; ++x) {
@@ -307,8 +294,8 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
         ld_col[x] = (cid % CH) * 8;
     }
     // A staged chunk: the 16 bytes as loaded (chunk positions past the row's whole chunks hold the row's last elements:
-    // load_chunk_unpadded, load_chunk_anyalign), except that rows of fewer than eight elements are fetched element by
-    // element and padded with zeroes.
+    // load_chunk_anyalign), except that rows of fewer than eight elements are fetched element by element and padded
+    // with zeroes.
     v4u kreg[NLD], vreg[NLD];
     auto gload = [&](const half_t* __restrict__ base, int tile, v4u (&reg)[NLD]) {
         const int kb0 = tile * BC;
@@ -316,8 +303,7 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
         for (int x = 0; x < NLD; ++x) {
             const int r = kb0 + ld_row[x];
             const half_t* __restrict__ rowp = base + (size_t)(r < Nk ? r : Nk - 1) * d;
-            if constexpr (kVec) reg[x] = load_chunk_unpadded<kVec, kFullD>(rowp, ld_col[x], d);
-            else reg[x] = !kEvery || d >= 8 ? load_chunk_anyalign(rowp, ld_col[x], d) : load_chunk<false, false>(rowp, ld_col[x], d);
+            reg[x] = d >= 8 ? load_chunk_anyalign(rowp, ld_col[x], d) : load_chunk<false, false>(rowp, ld_col[x], d);
         }
     };
     auto put_k = [&](int buf) {
@@ -337,7 +323,7 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
     // block x fetches whatever belongs into chunk 64 x + l (the pad chunk of a K row gets a copy of its neighbour).
     // Blocks go round the four waves; the odd K block goes to the waves that still have a block index left for it.
     // Rows shorter than the bucket: chunk positions past the row's whole chunks fetch the row's last 16 bytes (see
-    // load_chunk_unpadded, load_chunk_anyalign).
+    // load_chunk_anyalign): for K they meet zero columns of Q, for V they only reach rows of O^T that are never stored.
     const int row_bytes = kFullD ? D * 2 : d * 2;
     auto chunk_offset = [&](int c) { return kFullD ? c * 16 : (c * 8 + 8 <= d ? c * 16 : (d - 8) * 2); };
     uint32_t koff[C::NKX], voff[C::NVX];
