@@ -93,8 +93,8 @@ typedef struct flash_params {
      * feature and head dim, which is about 20 % slower.  No counterpart in the reference. */
     float *scores_out;
     /* Which tiled kernel serves the call, for A/B measurements and tests: 0 = the library chooses (by shape),
-     * 1 = the 4-wave kernel (128 query rows per work-group), 2 = the 8-wave ping-pong kernel (256 rows; needs d == 128
-     * in whole 16-byte rows and more than 128 query rows, and is ignored otherwise).  Any other value: FLASH_EINVAL.
+     * 1 = the 4-wave kernel (128 query rows per work-group), 2 = the 8-wave ping-pong kernel (256 rows; needs
+     * 96 < d <= 128, a positive scale and more than 128 query rows, and is ignored otherwise).  Any other value: FLASH_EINVAL.
      * The reference selects its kernel by template flags alone (src/main.cu:141-178) and has no such switch. */
     int kernel_hint;
     /* Optional debug output: when non-NULL, every work-group of the tiled kernel stores FLASH_STAMP_WORDS 64-bit words
