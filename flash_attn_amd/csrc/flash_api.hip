@@ -427,6 +427,9 @@ FLASH_EXPORT int flash_forward(const flash_params* p, void* stream)
     bool empty;
     int rc = validate(p, &empty);
     if (rc != FLASH_OK || empty) return rc;
+    // One query row per head takes the decode routes, unsplit: the streaming kernel, or the heads of a K/V head as the
+    // rows of one problem (the tiled kernel as it stands would give each head a 128-row work-group of its own).
+    if (p->Nq == 1) return run_splitkv(p, 1, static_cast<hipStream_t>(stream));
     if ((rc = device_usable()) != FLASH_OK) return rc;
     fa::FwdArgs a;
     fill_args(p, 1, &a);
@@ -474,7 +477,7 @@ FLASH_EXPORT int flash_stage_stamps_bytes(const flash_params* p, int split, size
     if (rc != FLASH_OK || empty) return rc;
     fa::FwdArgs a;
     fill_args(p, split ? resolve_splits(p) : 1, &a);
-    if (split && splitkv_route(p, &a) == kRouteStream) return FLASH_OK;
+    if ((split || p->Nq == 1) && splitkv_route(p, &a) == kRouteStream) return FLASH_OK;  // (flash_forward routes Nq == 1 too)
     *bytes = (size_t)tiled_groups(p, a) * FLASH_STAMP_WORDS * sizeof(uint64_t);
     return FLASH_OK;
 }
