@@ -247,6 +247,15 @@ int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode)
     const float partials = 8.0f * (float)slices * (float)p->Nq * (float)p->d / 4.2e6f;  // us per split
     const int shift = p->Nk - p->Nq;
     const bool masked = p->is_causal || wl >= 0 || wr >= 0;
+    // An unsplit launch may take the narrow instances (fa::fwd_uses_narrow): four times the work-groups, each wave
+    // walking a quarter of the tiles alone on its SIMD (x 1.15 per tile), two work-groups side by side per CU up to
+    // d = 32 and one above, 3 us for the launch and 4 us per work-group in a row on a CU (fitted to 12 shapes).
+    bool narrow = false;
+    if (!pp) {
+        fa::FwdArgs unsplit;
+        fill_args(p, 1, &unsplit);
+        narrow = fa::fwd_uses_narrow(unsplit, tiled_variant(p), every);
+    }
     int limit = FLASH_MAX_SPLITS;
     if (n_blocks < limit) limit = n_blocks;
     int best_s = 1, prev_per = -1;
@@ -287,6 +296,11 @@ int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode)
         const long long k = (groups + kNumCU - 1) / kNumCU;
         const float rho = k == 1 ? 1.0f : k == 2 ? rho2 : rho3;
         float t = ((float)k * a + b * ((float)tmax + (float)(k - 1) * (float)tiles / (float)groups)) / rho;
+        if (s == 1 && narrow) {
+            const long long kn = (4 * groups + kNumCU - 1) / kNumCU;
+            const float rhon = kn >= 2 && p->d <= 32 ? rho2 : 1.0f;
+            t = (3.0f + (float)kn * (a - 1.0f) + 1.15f * b * ((float)((tmax + 3) / 4) + (float)(kn - 1) * (float)tiles / (float)groups / 4.0f)) / rhon;
+        }
         if (s > 1) t += c0 + (float)s * (c1 + partials);
         if (s == 1 || t < best_t) {
             best_t = t;

@@ -110,13 +110,16 @@ constexpr float kLazyTau = 8.0f;
 // kVarKvOnce (with kVarVec, kVarFullD, no other feature): every K/V tile is requested by this work-group alone -- one row
 // block per slice and one query head per K/V head, the shape of a decode launch -- and its requests are non-temporal.
 // kVarEvery (with kVarAlibi and kVarDropout, without kVarVec): the instance that serves every request, see kEvery below.
+// kVarNarrow (D <= 64, unsplit launches): the four waves of a work-group share 32 query rows and take every fourth key
+// tile each, see kNarrow below.
 constexpr int kVarVec = 1, kVarAlibi = 2, kVarDropout = 4, kVarFullD = 8, kVarStamp = 16, kVarAlibiLeft = 32, kVarKvOnce = 64,
-              kVarEvery = 128;
+              kVarEvery = 128, kVarNarrow = 256;
 
 // work-groups per CU: three up to D = 64 (168 VGPRs), except for the instance that serves every request, which stages
 // its tiles through registers
 constexpr int fwd_groups_per_cu(int D, int NB, int VAR)
 {
+    if ((VAR & kVarNarrow) != 0) return 1;
     return NB == 1 ? (D <= 64 && (VAR & kVarEvery) == 0 ? 3 : 2) : 1;
 }
 
@@ -141,14 +144,26 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
     // the score dump among them.
     constexpr bool kEvery = (VAR & kVarEvery) != 0;
     static_assert(!kEvery || (!kVec && kAlibi && kDropout), "the instance that serves every request");
+    // Small problems -- fewer work-groups of 128 rows than half the CUs -- are bound by the chain of tiles that a
+    // work-group walks through one after the other.  The narrow instances cut that chain to a quarter: a work-group owns
+    // 32 query rows, all four waves hold those rows, and wave w takes the key tiles w, w + 4, w + 8, ... of the range on
+    // its own: it requests them into two LDS stages of its own (no work-group barrier inside the loop, every wave waits
+    // for its own requests only), and the four partial results are merged through LDS at the end like the partial results
+    // of a split -- in the same launch, where a split count of four would need the combine launch behind it.
+    constexpr bool kNarrow = (VAR & kVarNarrow) != 0;
+    static_assert(!kNarrow || (kDma && NB == 1 && D <= 64 && !kStamp && !kKvOnce), "narrow instances");
     constexpr int NSTG = kDma ? C::NSTG : 2;
+    constexpr int BRW = kNarrow ? 32 : C::BR;  // query rows per work-group
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    char* const Ks = smem;
-    char* const Vs = smem + NSTG * C::KBUF;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = wave_uniform(tid >> 6);
+    // tile buffers: of the work-group, or (narrow) of the wave
+    constexpr int kWaveLds = NSTG * (C::KBUF + C::VBUF);
+    const int lds_base = kNarrow ? wave * kWaveLds : 0;
+    char* const Ks = smem + lds_base;
+    char* const Vs = Ks + NSTG * C::KBUF;
     const int l32 = lane & 31;
     const int g = lane >> 5;
 
@@ -172,12 +187,13 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
     const int h = bh % a.H;
     const int Nq = a.Nq, Nk = a.Nk, d = kFullD ? D : a.d;
     const int shift = Nk - Nq;
-    const int q0 = m_block * C::BR;
+    const int q0 = m_block * BRW;
+    const int wave_row0 = kNarrow ? 0 : wave * C::RW;  // first row of the wave inside the work-group's block
 
     // ---- key range of the work-group (block pruning, src/flash_forward.h:39-48; split range, splitkv.h:40-43)
     int kmin = 0, kmax = Nk;
     {
-        const int last_row = (q0 + C::BR - 1 < Nq ? q0 + C::BR - 1 : Nq - 1) + shift;
+        const int last_row = (q0 + BRW - 1 < Nq ? q0 + BRW - 1 : Nq - 1) + shift;
         if (a.wl >= 0) kmin = max(0, q0 + shift - a.wl);
         if (a.causal) kmax = min(kmax, last_row + 1);
         if (a.wr >= 0) kmax = min(kmax, last_row + a.wr + 1);
@@ -190,7 +206,7 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
     const int tile_begin = kmin / BC;
     const int ntiles = kmax > kmin ? (kmax + BC - 1) / BC - tile_begin : 0;
     if (!kStamp && ntiles == 0) {  // (the instrumented twins take the long way and report their stages)
-        store_empty_rows(a, bh, split, q0, q0 + C::BR < Nq ? q0 + C::BR : Nq, tid, 256);
+        store_empty_rows(a, bh, split, q0, q0 + BRW < Nq ? q0 + BRW : Nq, tid, 256);
         return;
     }
 
@@ -199,7 +215,7 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
     float iif[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-        const int i = q0 + wave * C::RW + nb * 32 + l32;
+        const int i = q0 + wave_row0 + nb * 32 + l32;
         row_i[nb] = i;
         const int ii = (i < Nq ? i : Nq - 1) + shift;
         int l_ = 0, h_ = Nk - 1;
@@ -218,7 +234,7 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
     // test), nothing outside [lo_min, hi_max] is visible to any of them (a tile outside it is skipped by the wave)
     int lo_max, hi_min, lo_min, hi_max;
     {
-        const int first = q0 + wave * C::RW, last = first + C::RW - 1;
+        const int first = q0 + wave_row0, last = first + C::RW - 1;
         const int iif_ = (first < Nq ? first : Nq - 1) + shift, iil_ = (last < Nq ? last : Nq - 1) + shift;
         lo_max = lo_min = 0;
         hi_min = hi_max = Nk - 1;
@@ -326,33 +342,36 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
     // load_chunk_anyalign): for K they meet zero columns of Q, for V they only reach rows of O^T that are never stored.
     const int row_bytes = kFullD ? D * 2 : d * 2;
     auto chunk_offset = [&](int c) { return kFullD ? c * 16 : (c * 8 + 8 <= d ? c * 16 : (d - 8) * 2); };
-    uint32_t koff[C::NKX], voff[C::NVX];
-    int krow[C::NKX], vrow[C::NVX];
+    // (narrow: every block of a tile is the wave's own, and so is the buffer)
+    constexpr int NKX = kNarrow ? CH + 1 : C::NKX, NVX = kNarrow ? CH : C::NVX;
+    auto block_of = [&](int i) { return kNarrow ? i : wave + 4 * i; };
+    uint32_t koff[NKX], voff[NVX];
+    int krow[NKX], vrow[NVX];
     if constexpr (kDma) {
 #pragma unroll
-        for (int i = 0; i < C::NKX; ++i) {
-            const int q = 64 * (wave + 4 * i) + lane;
+        for (int i = 0; i < NKX; ++i) {
+            const int q = 64 * block_of(i) + lane;
             krow[i] = q / (CH + 1);
             const int col = q % (CH + 1);
             koff[i] = (uint32_t)(krow[i] * row_bytes + chunk_offset(col < CH ? col : CH - 1));
         }
 #pragma unroll
-        for (int i = 0; i < C::NVX; ++i) {
-            const int q = 64 * (wave + 4 * i) + lane;
+        for (int i = 0; i < NVX; ++i) {
+            const int q = 64 * block_of(i) + lane;
             vrow[i] = q / CH;
             const int c = q % CH;
             voff[i] = (uint32_t)(vrow[i] * row_bytes + chunk_offset(C::VSWZ ? c ^ (((vrow[i] >> 1) & 1) << 2) : c));
         }
     }
-    const bool k_extra = wave + 4 * (C::NKX - 1) <= CH;  // the last round of K blocks exists for this wave
+    const bool k_extra = kNarrow || wave + 4 * (NKX - 1) <= CH;  // the last round of K blocks exists for this wave
     auto dma_tile = [&](int tile, int stage) {
         // The tile's offset joins the scalar base address, so that a request of a whole tile needs no vector
         // arithmetic at all; only the last tile of a ragged sequence adjusts rows: keys past Nk re-read key Nk - 1
         // (their scores are masked).
         const size_t tb = (size_t)tile * (size_t)(BC * row_bytes);
         const int rows_left = Nk - tile * BC;  // >= 1
-        FA_LDS char* const kst = (FA_LDS char*)smem + stage * C::KBUF;
-        FA_LDS char* const vst = (FA_LDS char*)smem + NSTG * C::KBUF + stage * C::VBUF;
+        FA_LDS char* const kst = (FA_LDS char*)smem + lds_base + stage * C::KBUF;
+        FA_LDS char* const vst = (FA_LDS char*)smem + lds_base + NSTG * C::KBUF + stage * C::VBUF;
         const char* const Kb = reinterpret_cast<const char*>(Kbh) + tb;
         const char* const Vb = reinterpret_cast<const char*>(Vbh) + tb;
         auto issue = [&](auto ragged_c) {
@@ -362,19 +381,19 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
             int rows_left = Nk - tile * BC;
             if constexpr (kRagged) asm volatile("" : "+s"(rows_left));
 #pragma unroll
-            for (int i = 0; i < C::NKX; ++i) {
-                if (i == C::NKX - 1 && !k_extra) break;
+            for (int i = 0; i < NKX; ++i) {
+                if (i == NKX - 1 && !k_extra) break;
                 uint32_t o = koff[i];
                 if (kRagged && krow[i] >= rows_left) o -= (uint32_t)((krow[i] - rows_left + 1) * row_bytes);
-                if constexpr (kKvOnce) dma_kib_nt(Kb, o, kst + (wave + 4 * i) * 1024);
-                else dma_kib(Kb, o, kst + (wave + 4 * i) * 1024);
+                if constexpr (kKvOnce) dma_kib_nt(Kb, o, kst + block_of(i) * 1024);
+                else dma_kib(Kb, o, kst + block_of(i) * 1024);
             }
 #pragma unroll
-            for (int i = 0; i < C::NVX; ++i) {
+            for (int i = 0; i < NVX; ++i) {
                 uint32_t o = voff[i];
                 if (kRagged && vrow[i] >= rows_left) o -= (uint32_t)((vrow[i] - rows_left + 1) * row_bytes);
-                if constexpr (kKvOnce) dma_kib_nt(Vb, o, vst + (wave + 4 * i) * 1024);
-                else dma_kib(Vb, o, vst + (wave + 4 * i) * 1024);
+                if constexpr (kKvOnce) dma_kib_nt(Vb, o, vst + block_of(i) * 1024);
+                else dma_kib(Vb, o, vst + block_of(i) * 1024);
             }
         };
         if (rows_left >= BC) issue(std::false_type{});
@@ -383,8 +402,8 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
     // wait until at most the requests of one tile (the youngest) are still in flight / until none is
     auto dma_wait = [&](bool one_tile_in_flight) {
         if (!one_tile_in_flight) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        else if (k_extra) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(C::NKX + C::NVX) : "memory");
-        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(C::NKX + C::NVX - 1) : "memory");
+        else if (k_extra) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NKX + NVX) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NKX + NVX - 1) : "memory");
     };
 
     // ---- accumulators
@@ -710,7 +729,7 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
     // A wave whose rows all lie past Nq (fewer than 128 query rows: short prompts, or the heads of one K/V head decoding
     // together) only helps to stage the tiles, and so does any wave for a tile that none of its rows can see (the far
     // end of the causal diagonal block, the near end of a sliding window).
-    const bool wave_live = q0 + wave * C::RW < Nq;
+    const bool wave_live = q0 + wave_row0 < Nq;
     auto tile_math = [&](int t, int buf) {
         const int kb0 = (tile_begin + t) * BC;
         if (wave_live && kb0 <= hi_max && kb0 + BC - 1 >= lo_min) {
@@ -722,7 +741,31 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
             pv(buf, pf);
         }
     };
-    if constexpr (kDma) {
+    if constexpr (kNarrow) {
+        // Wave w walks the tiles w, w + 4, ... with two stages of its own: tile n + 2 is requested into the stage of
+        // tile n as soon as that tile's fragments have been read, and before tile n + 1 is touched its requests (older
+        // than those of tile n + 2) have been waited for.  No other wave reads or writes these buffers.
+        const int nt = wave < ntiles ? (ntiles - wave + 3) / 4 : 0;
+        static_assert(NKX + NVX <= 63, "vmcnt immediate");
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+            if (u < nt) dma_tile(tile_begin + wave + 4 * u, u);
+        read_slope();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        pin_q();
+        int buf = 0;
+        for (int n = 0; n < nt; ++n) {
+            tile_math(wave + 4 * n, buf);
+            if (n + 2 < nt) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the stage has been read
+                dma_tile(tile_begin + wave + 4 * (n + 2), buf);
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NKX + NVX) : "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
+            buf ^= 1;
+        }
+    } else if constexpr (kDma) {
         // Tile t + PF is requested when tile t starts (its stage was read last during tile t - 1, behind a barrier);
         // before the barrier that ends tile t, the requests of tile t + 1 have landed, those of t + 2 may be in flight.
         // Before tile 0 every stage is free: the prologue requests one tile per stage, so that the request which
@@ -730,7 +773,7 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
         // second time at the end of its first tile).
         constexpr int PF = NSTG - 1;
         static_assert(PF == 1 || PF == 2, "prefetch distance");
-        static_assert(C::NKX + C::NVX <= 15, "vmcnt immediate");
+        static_assert(NKX + NVX <= 63, "vmcnt immediate");
 #pragma unroll
         for (int u = 0; u < NSTG; ++u)
             if (u < ntiles) dma_tile(tile_begin + u, u);
@@ -783,6 +826,63 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
             }
             __syncthreads();
         }
+    }
+
+    if constexpr (kNarrow) {
+        // ---------------- merge of the four waves' partial results (same rows, disjoint keys), then O and LSE.
+        // Like the combine of split partials: weights 2^(m_w - M) on the row sums and on the unnormalised O.
+        __syncthreads();  // every wave is done with its tile buffers
+        float* const sm = reinterpret_cast<float*>(smem);  // [4][32] running maxima (log2 units)
+        float* const sl = sm + 4 * 32;                      // [4][32] row sums
+        float* const so = sl + 4 * 32;                      // [4][32][D] unnormalised O, by chunk position
+        static_assert((2 * 4 * 32 + 4 * 32 * D) * 4 <= 4 * kWaveLds, "merge buffers fit the tile buffers");
+        const float l = xhalf_sum(l_run[0]);
+        if (g == 0) {
+            sm[wave * 32 + l32] = m_ref[0];
+            sl[wave * 32 + l32] = l;
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+                const v4f o = {oacc[mb][0][4 * rg], oacc[mb][0][4 * rg + 1], oacc[mb][0][4 * rg + 2], oacc[mb][0][4 * rg + 3]};
+                *reinterpret_cast<v4f*>(so + (wave * 32 + l32) * D + 32 * mb + 8 * rg + 4 * g) = o;
+            }
+        __syncthreads();
+        // thread -> one row and D / 8 consecutive chunk positions of it
+        constexpr int CPT = D / 8;
+        const int row = tid >> 3, cp0 = (tid & 7) * CPT;
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) M = fmaxf(M, sm[w * 32 + row]);
+        const float Mu = (M == -INFINITY) ? 0.0f : M;
+        float L = 0.0f, wgt[4];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            wgt[w] = fast_exp2(sm[w * 32 + row] - Mu);
+            L += wgt[w] * sl[w * 32 + row];
+        }
+        const float inv = L > 0.0f ? (kDropout ? a.drop_rscale : 1.0f) / L : 0.0f;
+        const int gi = q0 + row;
+        if (gi < Nq) {
+            half_t* const op = a.O + ((size_t)bh * Nq + gi) * d;
+            const int cfull = d & ~7, rem = d & 7;
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) {
+                const int cc = cp0 + c;
+                float o = 0.0f;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) o = __builtin_fmaf(wgt[w], so[(w * 32 + row) * D + cc], o);
+                // column of chunk position cc: behind the row's whole chunks sit the columns d - 8 ... d - 1, of which
+                // the first 8 - d % 8 belong to the positions before
+                const int col = kFullD || cc < cfull ? cc : cc - (8 - rem);
+                const bool ok = kFullD || cc < cfull || (rem != 0 && cc < cfull + 8 && col >= cfull);
+                if (ok) op[col] = (half_t)(o * inv);
+            }
+            if ((tid & 7) == 0)
+                a.LSE[(size_t)bh * Nq + gi] = L > 0.0f ? __builtin_fmaf(M, kLn2, fast_log2(L) * kLn2) : -INFINITY;
+        }
+        return;
     }
 
     // ---------------- epilogue: normalise once, store O (fp16) + LSE, or the fp32 split partials
@@ -947,6 +1047,37 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
 // The instances of a bucket: {d == bucket, d % 8 == 0} x {plain, ALiBi, ALiBi with every visible key at or left of its
 // row, dropout, both}, for rows at any alignment (d % 8 != 0) {plain, ALiBi, dropout, both}, and the one that serves
 // every other request.  ST = kVarStamp selects their instrumented twins (debug time stamps).
+// The narrow instances (kNarrow in fwd_kernel): unsplit launches without ALiBi and dropout up to d = 64 that would
+// occupy at most half the CUs with work-groups of 128 rows, each of them with 16 key tiles or more ahead of it (8 where
+// they occupy a quarter of the CUs).  Measured against the 128-row instances, same box: B1 H8 N1021 d31 (the reference's
+// own run) 14.2 -> 11.8 us, B1 H8 N1024 d64 15.0 -> 10.2, B1 H8 N2048 d64 causal 27.3 -> 17.8, B1 H1 N2048 d32 causal
+// 22.2 -> 10.5, B1 H4 N4096 d64 50.1 -> 38.0; with 128 work-groups of 8 tiles (B1 H32 N512 d64) 10.3 -> 11.8, hence the limit.
+inline bool fwd_uses_narrow(const FwdArgs& a, int variant, bool every)
+{
+    if (every || (variant & (kVarAlibi | kVarDropout)) != 0 || a.num_splits != 1 || a.stamps != nullptr || a.kernel_hint != 0) return false;
+    const long long groups = (long long)a.B * a.H * ((a.Nq + 127) / 128);
+    if (a.d > 64 || 2 * groups > kNumCus) return false;
+    const int keys = 4 * groups <= kNumCus ? 512 : 1024;  // visible keys per row that make the chain worth cutting
+    return a.Nk >= keys && (a.wl < 0 || a.wl >= keys - 64);
+}
+
+template <int D, int VAR>
+inline hipError_t launch_fwd_narrow_instance(const FwdArgs& a, hipStream_t st)
+{
+    using C = FwdCfg<D, 1>;
+    auto kern = fwd_kernel<D, 1, VAR | kVarNarrow>;
+    static DeviceFlags attr_done;  // per instantiation and device
+    constexpr int smem = 4 * C::NSTG * (C::KBUF + C::VBUF);  // two stages per wave
+    if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, attr_done); e != hipSuccess) return e;
+    FwdArgs b = a;
+    b.Tr = (a.Nq + 31) / 32;
+    const long long groups = (long long)b.Tr * a.B * a.H;
+    set_slice_order(b, b.Tr, kNumCus);
+    b.split_rotate = 0;
+    b.snake_end = snake_end_for(groups, kNumCus);
+    return launch_kernel(kern, dim3((unsigned)groups), dim3(256), smem, st, b);
+}
+
 // requests that only the instance which serves every request takes (kEvery in fwd_kernel)
 inline bool fwd_needs_every_instance(const FwdArgs& a, int variant)
 {
@@ -959,6 +1090,13 @@ inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
     hipError_t e;
     const int feat = variant & (kVarAlibi | kVarDropout);
     constexpr int AL = kVarAlibi | kVarAlibiLeft;  // ALiBi with no visible key right of its row
+    if constexpr (D <= 64 && ST == 0) {
+        if (fwd_uses_narrow(a, variant, fwd_needs_every_instance(a, variant))) {
+            if (!(variant & kVarVec)) return (int)launch_fwd_narrow_instance<D, 0>(a, st);
+            if (a.d == D) return (int)launch_fwd_narrow_instance<D, kVarVec | kVarFullD>(a, st);
+            return (int)launch_fwd_narrow_instance<D, kVarVec>(a, st);
+        }
+    }
     if (!(variant & kVarVec)) {
         // rows at any alignment: plain, ALiBi, dropout, both, and one more with both features compiled in (slope 0 /
         // threshold 0 make them identities) for every other request: a non-positive scale (its ALiBi step is where the

@@ -101,6 +101,42 @@ def test_8wave_kernel_on_shorter_rows(fa, oracle, d):
             assert np.array_equal(km.cpu().numpy()[..., vis], keep[..., vis]), f"d={d}"
 
 
+# Small unsplit problems up to d = 64 (the reference's own run among them) take work-groups of 32 rows whose four waves
+# walk every fourth key tile each and merge their results through LDS.  Ragged row and key counts (rows that are not a
+# multiple of 32, a last tile of one key), causal rows whose upper waves get no tile at all, Nq != Nk in both directions
+# (leading row blocks without a visible key), wide windows, grouped K/V heads, head dims in both buckets: whole chunks,
+# the bucket width, every alignment.  kernel_hint = KERNEL_4WAVE runs the 128-row instances on the same request.
+@pytest.mark.parametrize("B,H,Hk,Nq,Nk,d,kw", [
+    (1, 8, 8, 1021, 1021, 31, dict()),                      # the reference's checked-in run (src/main.cu:39-49)
+    (1, 8, 8, 1021, 1021, 31, dict(causal=True)),
+    (1, 4, 4, 1000, 1025, 64, dict(causal=True)),
+    (2, 4, 2, 777, 777, 64, dict()),
+    (1, 6, 3, 300, 2000, 40, dict(window=(700, 100))),
+    (1, 3, 3, 900, 600, 63, dict(causal=True)),             # rows 0 ... 299 see nothing
+    (1, 2, 1, 33, 4097, 17, dict()),
+    (2, 2, 2, 515, 515, 56, dict(causal=True, window=(600, -1))),
+    (1, 5, 5, 640, 640, 32, dict(window=(-1, 64))),
+    (1, 4, 4, 1, 3000, 20, dict(dropout_p=0.0)),            # one row: the decode kernel, not these instances
+])
+def test_narrow_instances(fa, oracle, B, H, Hk, Nq, Nk, d, kw):
+    import torch
+    q = randn_f16_gpu((B, H, Nq, d), 41)
+    k = randn_f16_gpu((B, Hk, Nk, d), 42)
+    v = randn_f16_gpu((B, Hk, Nk, d), 43)
+    kr, vr = (t.repeat_interleave(H // Hk, dim=1).contiguous() for t in (k, v))
+    okw = {x: kw[x] for x in ("causal", "window") if x in kw}
+    O, L = oracle_forward_batched(oracle, q, kr, vr, **okw)
+    o = torch.full((B, H, Nq, d), float("nan"), dtype=torch.float16, device="cuda")
+    lse = torch.full((B, H, Nq), float("nan"), dtype=torch.float32, device="cuda")
+    fa.flash_forward(q, k, v, out=o, lse=lse, **kw)
+    check_o_lse(o, lse, O, L, f"32-row work-groups {(B, H, Hk, Nq, Nk, d)} {sorted(kw)}")
+    o1, lse1 = fa.flash_forward_splitkv(q, k, v, num_splits=1, **kw)
+    assert torch.equal(o, o1) and torch.equal(lse, lse1)
+    o4, lse4 = fa.flash_forward(q, k, v, kernel_hint=fa.KERNEL_4WAVE, **kw)
+    check_o_lse(o4, lse4, O, L, f"128-row work-groups {(B, H, Hk, Nq, Nk, d)} {sorted(kw)}")
+    assert torch.allclose(o.float(), o4.float(), atol=2e-3, rtol=1e-2)
+
+
 # sequence lengths around the tile sizes (64-key tiles, 128-row groups); 1021 is the reference's checked-in seq_len
 @pytest.mark.parametrize("N", [1, 2, 31, 63, 64, 65, 127, 128, 129, 191, 257, 1000, 1021])
 def test_ragged_lengths(fa, oracle, N):
@@ -303,7 +339,7 @@ def test_split_index_rotation(fa, oracle, H, S):
 @pytest.mark.parametrize("B,H,Nq,Nk,d,causal,want", [
     (1, 8, 512, 32768, 128, False, 16),   # long keys, small batch: two work-groups per CU
     (1, 32, 128, 16384, 128, True, 8),    # causal with Nq < Nk: every split holds visible keys
-    (1, 4, 2048, 2048, 63, False, 4),     # rows at any alignment
+    (1, 4, 2048, 2048, 100, False, 4),    # rows at any alignment
     (1, 2, 8192, 8192, 64, True, None),   # causal, one work-group per CU at most: split for the heaviest row block
     (1, 40, 128, 8192, 128, False, 6),
 ])
