@@ -1047,14 +1047,14 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
 // The instances of a bucket: {d == bucket, d % 8 == 0} x {plain, ALiBi, ALiBi with every visible key at or left of its
 // row, dropout, both}, for rows at any alignment (d % 8 != 0) {plain, ALiBi, dropout, both}, and the one that serves
 // every other request.  ST = kVarStamp selects their instrumented twins (debug time stamps).
-// The narrow instances (kNarrow in fwd_kernel): unsplit launches without ALiBi and dropout up to d = 64 that would
+// The narrow instances (kNarrow in fwd_kernel): unsplit launches up to d = 64 that would
 // occupy at most half the CUs with work-groups of 128 rows, each of them with 16 key tiles or more ahead of it (8 where
 // they occupy a quarter of the CUs).  Measured against the 128-row instances, same box: B1 H8 N1021 d31 (the reference's
 // own run) 14.2 -> 11.8 us, B1 H8 N1024 d64 15.0 -> 10.2, B1 H8 N2048 d64 causal 27.3 -> 17.8, B1 H1 N2048 d32 causal
 // 22.2 -> 10.5, B1 H4 N4096 d64 50.1 -> 38.0; with 128 work-groups of 8 tiles (B1 H32 N512 d64) 10.3 -> 11.8, hence the limit.
 inline bool fwd_uses_narrow(const FwdArgs& a, int variant, bool every)
 {
-    if (every || (variant & (kVarAlibi | kVarDropout)) != 0 || a.num_splits != 1 || a.stamps != nullptr || a.kernel_hint != 0) return false;
+    if (every || a.num_splits != 1 || a.stamps != nullptr || a.kernel_hint != 0) return false;
     const long long groups = (long long)a.B * a.H * ((a.Nq + 127) / 128);
     if (a.d > 64 || 2 * groups > kNumCus) return false;
     const int keys = 4 * groups <= kNumCus ? 512 : 1024;  // visible keys per row that make the chain worth cutting
@@ -1092,6 +1092,11 @@ inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
     constexpr int AL = kVarAlibi | kVarAlibiLeft;  // ALiBi with no visible key right of its row
     if constexpr (D <= 64 && ST == 0) {
         if (fwd_uses_narrow(a, variant, fwd_needs_every_instance(a, variant))) {
+            // plain: by row length like the others; with ALiBi or dropout: the instances for rows at any alignment,
+            // which serve every row length from eight elements on
+            if (feat == kVarAlibi) return (int)launch_fwd_narrow_instance<D, kVarAlibi>(a, st);
+            if (feat == kVarDropout) return (int)launch_fwd_narrow_instance<D, kVarDropout>(a, st);
+            if (feat != 0) return (int)launch_fwd_narrow_instance<D, kVarAlibi | kVarDropout>(a, st);
             if (!(variant & kVarVec)) return (int)launch_fwd_narrow_instance<D, 0>(a, st);
             if (a.d == D) return (int)launch_fwd_narrow_instance<D, kVarVec | kVarFullD>(a, st);
             return (int)launch_fwd_narrow_instance<D, kVarVec>(a, st);

@@ -117,6 +117,10 @@ def test_8wave_kernel_on_shorter_rows(fa, oracle, d):
     (2, 2, 2, 515, 515, 56, dict(causal=True, window=(600, -1))),
     (1, 5, 5, 640, 640, 32, dict(window=(-1, 64))),
     (1, 4, 4, 1, 3000, 20, dict(dropout_p=0.0)),            # one row: the decode kernel, not these instances
+    (1, 4, 2, 700, 700, 64, dict(causal=True, alibi=True)),
+    (1, 3, 3, 500, 1100, 31, dict(alibi=True)),
+    (1, 2, 2, 600, 600, 48, dict(causal=True, dropout_p=0.2, seed=5, offset=77)),
+    (2, 2, 1, 333, 900, 27, dict(window=(800, 30), alibi=True, dropout_p=0.5, seed=2 ** 35, offset=1)),
 ])
 def test_narrow_instances(fa, oracle, B, H, Hk, Nq, Nk, d, kw):
     import torch
@@ -124,7 +128,26 @@ def test_narrow_instances(fa, oracle, B, H, Hk, Nq, Nk, d, kw):
     k = randn_f16_gpu((B, Hk, Nk, d), 42)
     v = randn_f16_gpu((B, Hk, Nk, d), 43)
     kr, vr = (t.repeat_interleave(H // Hk, dim=1).contiguous() for t in (k, v))
+    kw = dict(kw)
     okw = {x: kw[x] for x in ("causal", "window") if x in kw}
+    if kw.pop("alibi", False):
+        sl, sl_t = _slopes(oracle, H)
+        kw["alibi_slopes"], okw["slopes"] = sl_t, sl
+    p = kw.get("dropout_p", 0.0)
+    if p > 0.0:
+        keep = oracle.dropout_keep_mask(kw["seed"], kw["offset"], p, B, H, Nq, Nk)
+        okw.update(keep_mask=torch.from_numpy(keep), p_drop=p)
+        _, _, km = fa.flash_forward(q, k, v, return_keep_mask=True, **kw)
+        i, j = np.arange(Nq)[:, None] + (Nk - Nq), np.arange(Nk)[None, :]
+        wl, wr = kw.get("window", (-1, -1))
+        vis = np.ones((Nq, Nk), dtype=bool)
+        if kw.get("causal"):
+            vis &= j <= i
+        if wl >= 0:
+            vis &= j >= i - wl
+        if wr >= 0:
+            vis &= j <= i + wr
+        assert np.array_equal(km.cpu().numpy()[..., vis], keep[..., vis])
     O, L = oracle_forward_batched(oracle, q, kr, vr, **okw)
     o = torch.full((B, H, Nq, d), float("nan"), dtype=torch.float16, device="cuda")
     lse = torch.full((B, H, Nq), float("nan"), dtype=torch.float32, device="cuda")
