@@ -249,7 +249,7 @@ int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode)
     const bool masked = p->is_causal || wl >= 0 || wr >= 0;
     // An unsplit launch may take the narrow instances (fa::fwd_uses_narrow): four times the work-groups, each wave
     // walking a quarter of the tiles alone on its SIMD (x 1.15 per tile), two work-groups side by side per CU up to
-    // d = 32 and one above, 3 us for the launch and 4 us per work-group in a row on a CU (fitted to 12 shapes).
+    // d = 32 and one in a row above, 3 us for the launch and 4 us per work-group in a row on a CU (fitted to 12 shapes).
     bool narrow = false;
     if (!pp) {
         fa::FwdArgs unsplit;

@@ -110,8 +110,8 @@ constexpr float kLazyTau = 8.0f;
 // kVarKvOnce (with kVarVec, kVarFullD, no other feature): every K/V tile is requested by this work-group alone -- one row
 // block per slice and one query head per K/V head, the shape of a decode launch -- and its requests are non-temporal.
 // kVarEvery (with kVarAlibi and kVarDropout, without kVarVec): the instance that serves every request, see kEvery below.
-// kVarNarrow (D <= 64, unsplit launches): the four waves of a work-group share 32 query rows and take every fourth key
-// tile each, see kNarrow below.
+// kVarNarrow (unsplit launches): the four waves of a work-group share 32 query rows and take every fourth key tile
+// each, see kNarrow below.
 constexpr int kVarVec = 1, kVarAlibi = 2, kVarDropout = 4, kVarFullD = 8, kVarStamp = 16, kVarAlibiLeft = 32, kVarKvOnce = 64,
               kVarEvery = 128, kVarNarrow = 256;
 
@@ -147,12 +147,13 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
     // Small problems -- fewer work-groups of 128 rows than half the CUs -- are bound by the chain of tiles that a
     // work-group walks through one after the other.  The narrow instances cut that chain to a quarter: a work-group owns
     // 32 query rows, all four waves hold those rows, and wave w takes the key tiles w, w + 4, w + 8, ... of the range on
-    // its own: it requests them into two LDS stages of its own (no work-group barrier inside the loop, every wave waits
+    // its own: it requests them into LDS stages of its own (no work-group barrier inside the loop, every wave waits
     // for its own requests only), and the four partial results are merged through LDS at the end like the partial results
     // of a split -- in the same launch, where a split count of four would need the combine launch behind it.
     constexpr bool kNarrow = (VAR & kVarNarrow) != 0;
-    static_assert(!kNarrow || (kDma && NB == 1 && D <= 64 && !kStamp && !kKvOnce), "narrow instances");
-    constexpr int NSTG = kDma ? C::NSTG : 2;
+    static_assert(!kNarrow || (kDma && NB == 1 && !kStamp && !kKvOnce), "narrow instances");
+    // (narrow: two stages per wave up to D = 64, one above: four waves' tiles of 26 / 33 KiB)
+    constexpr int NSTG = kNarrow ? (D <= 64 ? 2 : 1) : kDma ? C::NSTG : 2;
     constexpr int BRW = kNarrow ? 32 : C::BR;  // query rows per work-group
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -364,7 +365,7 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
         }
     }
     const bool k_extra = kNarrow || wave + 4 * (NKX - 1) <= CH;  // the last round of K blocks exists for this wave
-    auto dma_tile = [&](int tile, int stage) {
+    auto dma_tile_parts = [&](int tile, int stage, auto k_part, auto v_part) {
         // The tile's offset joins the scalar base address, so that a request of a whole tile needs no vector
         // arithmetic at all; only the last tile of a ragged sequence adjusts rows: keys past Nk re-read key Nk - 1
         // (their scores are masked).
@@ -382,7 +383,7 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
             if constexpr (kRagged) asm volatile("" : "+s"(rows_left));
 #pragma unroll
             for (int i = 0; i < NKX; ++i) {
-                if (i == NKX - 1 && !k_extra) break;
+                if (!decltype(k_part)::value || (i == NKX - 1 && !k_extra)) break;
                 uint32_t o = koff[i];
                 if (kRagged && krow[i] >= rows_left) o -= (uint32_t)((krow[i] - rows_left + 1) * row_bytes);
                 if constexpr (kKvOnce) dma_kib_nt(Kb, o, kst + block_of(i) * 1024);
@@ -390,6 +391,7 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
             }
 #pragma unroll
             for (int i = 0; i < NVX; ++i) {
+                if (!decltype(v_part)::value) break;
                 uint32_t o = voff[i];
                 if (kRagged && vrow[i] >= rows_left) o -= (uint32_t)((vrow[i] - rows_left + 1) * row_bytes);
                 if constexpr (kKvOnce) dma_kib_nt(Vb, o, vst + block_of(i) * 1024);
@@ -399,6 +401,7 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
         if (rows_left >= BC) issue(std::false_type{});
         else issue(std::true_type{});
     };
+    auto dma_tile = [&](int tile, int stage) { dma_tile_parts(tile, stage, std::true_type{}, std::true_type{}); };
     // wait until at most the requests of one tile (the youngest) are still in flight / until none is
     auto dma_wait = [&](bool one_tile_in_flight) {
         if (!one_tile_in_flight) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -748,22 +751,50 @@ __global__ void __launch_bounds__(256, fwd_groups_per_cu(D, NB, VAR)) fwd_kernel
         const int nt = wave < ntiles ? (ntiles - wave + 3) / 4 : 0;
         static_assert(NKX + NVX <= 63, "vmcnt immediate");
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+        for (int u = 0; u < NSTG; ++u)
             if (u < nt) dma_tile(tile_begin + wave + 4 * u, u);
         read_slope();
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         pin_q();
-        int buf = 0;
-        for (int n = 0; n < nt; ++n) {
-            tile_math(wave + 4 * n, buf);
-            if (n + 2 < nt) {
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the stage has been read
-                dma_tile(tile_begin + wave + 4 * (n + 2), buf);
-                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NKX + NVX) : "memory");
-            } else {
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if constexpr (NSTG == 2) {
+            int buf = 0;
+            for (int n = 0; n < nt; ++n) {
+                tile_math(wave + 4 * n, buf);
+                if (n + 2 < nt) {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the stage has been read
+                    dma_tile(tile_begin + wave + 4 * (n + 2), buf);
+                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NKX + NVX) : "memory");
+                } else {
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                }
+                buf ^= 1;
             }
-            buf ^= 1;
+        } else {
+            // One stage: K(n + 1) is requested as soon as the scores of tile n are out of the K buffer, V(n + 1) as soon
+            // as the V buffer has been read; each is waited for right before its first use, the younger request of the
+            // other tensor staying in flight.
+            for (int n = 0; n < nt; ++n) {
+                const int kb0 = (tile_begin + wave + 4 * n) * BC;
+                const bool live = wave_live && kb0 <= hi_max && kb0 + BC - 1 >= lo_min;
+                const bool more = n + 1 < nt;
+                v16f s[2][NB];
+                v8h pf[2][2][NB];
+                if (live) qk(0, s);
+                if (more) {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    dma_tile_parts(tile_begin + wave + 4 * (n + 1), 0, std::true_type{}, std::false_type{});
+                }
+                if (live) softmax((kb0 < lo_max ? 1 : 0) | (kb0 + BC - 1 > hi_min ? 2 : 0), kb0, s, pf);
+                // V(n): older than the K request just issued
+                if (more) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NKX) : "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                if (live) pv(0, pf);
+                if (more) {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    dma_tile_parts(tile_begin + wave + 4 * (n + 1), 0, std::false_type{}, std::true_type{});
+                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NVX) : "memory");  // K(n + 1) is there
+                }
+            }
         }
     } else if constexpr (kDma) {
         // Tile t + PF is requested when tile t starts (its stage was read last during tile t - 1, behind a barrier);
@@ -1047,16 +1078,17 @@ inline hipError_t launch_fwd_instance(const FwdArgs& a, hipStream_t st)
 // The instances of a bucket: {d == bucket, d % 8 == 0} x {plain, ALiBi, ALiBi with every visible key at or left of its
 // row, dropout, both}, for rows at any alignment (d % 8 != 0) {plain, ALiBi, dropout, both}, and the one that serves
 // every other request.  ST = kVarStamp selects their instrumented twins (debug time stamps).
-// The narrow instances (kNarrow in fwd_kernel): unsplit launches up to d = 64 that would
+// The narrow instances (kNarrow in fwd_kernel): unsplit launches that would
 // occupy at most half the CUs with work-groups of 128 rows, each of them with 16 key tiles or more ahead of it (8 where
 // they occupy a quarter of the CUs).  Measured against the 128-row instances, same box: B1 H8 N1021 d31 (the reference's
 // own run) 14.2 -> 11.8 us, B1 H8 N1024 d64 15.0 -> 10.2, B1 H8 N2048 d64 causal 27.3 -> 17.8, B1 H1 N2048 d32 causal
-// 22.2 -> 10.5, B1 H4 N4096 d64 50.1 -> 38.0; with 128 work-groups of 8 tiles (B1 H32 N512 d64) 10.3 -> 11.8, hence the limit.
+// 22.2 -> 10.5, B1 H4 N4096 d64 50.1 -> 38.0, B1 H8 N1024 d128 20.9 -> 14.3; with 128 work-groups of 8 tiles (B1 H32
+// N512 d64) 10.3 -> 11.8, hence the limit.
 inline bool fwd_uses_narrow(const FwdArgs& a, int variant, bool every)
 {
     if (every || a.num_splits != 1 || a.stamps != nullptr || a.kernel_hint != 0) return false;
     const long long groups = (long long)a.B * a.H * ((a.Nq + 127) / 128);
-    if (a.d > 64 || 2 * groups > kNumCus) return false;
+    if (2 * groups > kNumCus) return false;
     const int keys = 4 * groups <= kNumCus ? 512 : 1024;  // visible keys per row that make the chain worth cutting
     return a.Nk >= keys && (a.wl < 0 || a.wl >= keys - 64);
 }
@@ -1067,7 +1099,7 @@ inline hipError_t launch_fwd_narrow_instance(const FwdArgs& a, hipStream_t st)
     using C = FwdCfg<D, 1>;
     auto kern = fwd_kernel<D, 1, VAR | kVarNarrow>;
     static DeviceFlags attr_done;  // per instantiation and device
-    constexpr int smem = 4 * C::NSTG * (C::KBUF + C::VBUF);  // two stages per wave
+    constexpr int smem = 4 * (D <= 64 ? 2 : 1) * (C::KBUF + C::VBUF);  // two stages per wave up to D = 64, one above
     if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, attr_done); e != hipSuccess) return e;
     FwdArgs b = a;
     b.Tr = (a.Nq + 31) / 32;
@@ -1090,7 +1122,7 @@ inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
     hipError_t e;
     const int feat = variant & (kVarAlibi | kVarDropout);
     constexpr int AL = kVarAlibi | kVarAlibiLeft;  // ALiBi with no visible key right of its row
-    if constexpr (D <= 64 && ST == 0) {
+    if constexpr (ST == 0) {
         if (fwd_uses_narrow(a, variant, fwd_needs_every_instance(a, variant))) {
             // plain: by row length like the others; with ALiBi or dropout: the instances for rows at any alignment,
             // which serve every row length from eight elements on

@@ -133,13 +133,15 @@ def test_split_resolution_and_workspace(fa):
     # automatic choice (num_splits <= 0) for Nq > 1: the count with the lowest estimated time (work-groups on the fullest
     # CU, prologue / epilogue per work-group, partial results per split).  The reference's checked-in shape
     # B=1,H=8,N=1021,d=31 stays whole (64 work-groups of 16 short tiles: measured 14.4 us, 4 splits 16.3), and so does
-    # twice that batch (14.4 us, 4 splits 22.0); so do half as many slices of twice the length at d = 63, where the
-    # work-groups of 32 rows whose waves share out the key tiles serve the unsplit launch, while at d = 100, beyond those
-    # instances, the same shape splits 4 ways; the prefill benchmark shapes stay unsplit
+    # twice that batch (14.4 us, 4 splits 22.0); so do half as many slices of twice the length, where work-groups of 32
+    # rows whose waves share out the key tiles serve the unsplit launch (with the 128-row instances it would split 4
+    # ways), while few rows in front of long keys still split; the prefill benchmark shapes stay unsplit
     assert fa.resolve_splits(1, 8, 1021, 1021, 31, 0) == 1
     assert fa.resolve_splits(2, 8, 1021, 1021, 31, 0) == 1
     assert fa.resolve_splits(1, 4, 2048, 2048, 63, 0) == 1
-    assert fa.resolve_splits(1, 4, 2048, 2048, 100, 0) == 4
+    assert fa.resolve_splits(1, 4, 2048, 2048, 100, 0) == 1
+    assert fa.resolve_splits(1, 4, 2048, 2048, 100, 0, kernel_hint=fa.KERNEL_4WAVE) == 4
+    assert fa.resolve_splits(1, 8, 200, 8000, 100, 0) == 16
     assert fa.resolve_splits(4, 16, 2048, 2048, 128, 0) == 1
     assert fa.resolve_splits(4, 16, 2048, 2048, 128, 0, causal=True) == 1
     assert fa.resolve_splits(8, 32, 1000, 1000, 96, 0, causal=True) == 1
@@ -152,9 +154,9 @@ def test_split_resolution_and_workspace(fa):
     assert fa.resolve_splits(2, 4, 300, 20000, 96, 0) == 10
     # 10 key blocks, 52 work-groups: 4 splits of 3 blocks fill 208 of 256 CUs (the reference's rule only looks at counts
     # with 1280 % (128 s) == 0 and would take 10 splits of one block)
-    assert fa.resolve_splits(1, 52, 100, 1280, 96, 0) == 4
-    # (up to d = 64 the unsplit launch has work-groups of 32 rows whose waves share out the key tiles, and wins:
-    # measured 11.3 us against 15.1 us in 4 splits)
+    assert fa.resolve_splits(1, 52, 100, 1280, 64, 0, kernel_hint=fa.KERNEL_4WAVE) == 4
+    # (left to itself the library serves this launch unsplit with work-groups of 32 rows whose waves share out the key
+    # tiles: measured 11.3 us against 15.1 us in 4 splits)
     assert fa.resolve_splits(1, 52, 100, 1280, 64, 0) == 1
     assert fa.num_splits_heuristic(52, 256, 10, 128, 1280) == 10
     # causal with one work-group per CU at most: split along the keys when the heaviest row block is long enough to

@@ -101,7 +101,7 @@ def test_8wave_kernel_on_shorter_rows(fa, oracle, d):
             assert np.array_equal(km.cpu().numpy()[..., vis], keep[..., vis]), f"d={d}"
 
 
-# Small unsplit problems up to d = 64 (the reference's own run among them) take work-groups of 32 rows whose four waves
+# Small unsplit problems (the reference's own run among them) take work-groups of 32 rows whose four waves
 # walk every fourth key tile each and merge their results through LDS.  Ragged row and key counts (rows that are not a
 # multiple of 32, a last tile of one key), causal rows whose upper waves get no tile at all, Nq != Nk in both directions
 # (leading row blocks without a visible key), wide windows, grouped K/V heads, head dims in both buckets: whole chunks,
@@ -117,6 +117,13 @@ def test_8wave_kernel_on_shorter_rows(fa, oracle, d):
     (2, 2, 2, 515, 515, 56, dict(causal=True, window=(600, -1))),
     (1, 5, 5, 640, 640, 32, dict(window=(-1, 64))),
     (1, 4, 4, 1, 3000, 20, dict(dropout_p=0.0)),            # one row: the decode kernel, not these instances
+    # above d = 64 a wave has one LDS stage and requests K and V of its next tile separately
+    (1, 8, 8, 1024, 1024, 128, dict(causal=True)),
+    (1, 4, 2, 777, 1100, 100, dict(window=(1000, 20))),
+    (2, 2, 2, 515, 515, 96, dict(alibi=True)),
+    (1, 3, 3, 900, 600, 127, dict(causal=True)),
+    (1, 2, 2, 600, 700, 120, dict(causal=True, dropout_p=0.3, seed=9, offset=2)),
+    (1, 2, 1, 40, 5000, 72, dict()),
     (1, 4, 2, 700, 700, 64, dict(causal=True, alibi=True)),
     (1, 3, 3, 500, 1100, 31, dict(alibi=True)),
     (1, 2, 2, 600, 600, 48, dict(causal=True, dropout_p=0.2, seed=5, offset=77)),
@@ -362,7 +369,7 @@ def test_split_index_rotation(fa, oracle, H, S):
 @pytest.mark.parametrize("B,H,Nq,Nk,d,causal,want", [
     (1, 8, 512, 32768, 128, False, 16),   # long keys, small batch: two work-groups per CU
     (1, 32, 128, 16384, 128, True, 8),    # causal with Nq < Nk: every split holds visible keys
-    (1, 4, 2048, 2048, 100, False, 4),    # rows at any alignment
+    (1, 8, 200, 8000, 100, False, 16),    # rows at any alignment
     (1, 2, 8192, 8192, 64, True, None),   # causal, one work-group per CU at most: split for the heaviest row block
     (1, 40, 128, 8192, 128, False, 6),
 ])
