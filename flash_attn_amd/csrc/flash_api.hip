@@ -248,8 +248,8 @@ int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode)
     const int shift = p->Nk - p->Nq;
     const bool masked = p->is_causal || wl >= 0 || wr >= 0;
     // An unsplit launch may take the narrow instances (fa::fwd_uses_narrow): four times the work-groups, each wave
-    // walking a quarter of the tiles alone on its SIMD (x 1.15 per tile), two work-groups side by side per CU up to
-    // d = 32 and one in a row above, 3 us for the launch and 4 us per work-group in a row on a CU (fitted to 12 shapes).
+    // walking a quarter of the tiles alone on its SIMD, two work-groups side by side per CU up to d = 32 and one in a
+    // row above, 3 us for the launch and 4 us per work-group in a row on a CU (fitted to 12 shapes).
     bool narrow = false;
     if (!pp) {
         fa::FwdArgs unsplit;
@@ -297,9 +297,15 @@ int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode)
         const float rho = k == 1 ? 1.0f : k == 2 ? rho2 : rho3;
         float t = ((float)k * a + b * ((float)tmax + (float)(k - 1) * (float)tiles / (float)groups)) / rho;
         if (s == 1 && narrow) {
-            const long long kn = (4 * groups + kNumCU - 1) / kNumCU;
+            // 32-row work-groups with a visible key, and the time per tile of a wave on its own, measured: x 1.15 with
+            // two LDS stages per wave (d <= 64); with one, where the next tile's requests are only partly hidden, x 1.3 at
+            // d = 96, x 1.6 at d = 128 and x 2.1 for rows shorter than the bucket; work-groups that follow another on
+            // their CU find their tiles in L2 and take half of that
+            const long long gn = (groups * ((p->Nq + 31) / 32) + Tr - 1) / Tr;
+            const long long kn = (gn + kNumCU - 1) / kNumCU;
             const float rhon = kn >= 2 && p->d <= 32 ? rho2 : 1.0f;
-            t = (3.0f + (float)kn * (a - 1.0f) + 1.15f * b * ((float)((tmax + 3) / 4) + (float)(kn - 1) * (float)tiles / (float)groups / 4.0f)) / rhon;
+            const float bn = (p->d <= 64 ? 1.15f : !dma ? 2.1f : bucket == 3 ? 1.3f : 1.6f) * b;
+            t = (3.0f + (float)kn * (a - 1.0f) + bn * ((float)((tmax + 3) / 4) + 0.5f * (float)(kn - 1) * (float)tiles / (float)groups / 4.0f)) / rhon;
         }
         if (s > 1) t += c0 + (float)s * (c1 + partials);
         if (s == 1 || t < best_t) {

@@ -133,14 +133,15 @@ def test_split_resolution_and_workspace(fa):
     # automatic choice (num_splits <= 0) for Nq > 1: the count with the lowest estimated time (work-groups on the fullest
     # CU, prologue / epilogue per work-group, partial results per split).  The reference's checked-in shape
     # B=1,H=8,N=1021,d=31 stays whole (64 work-groups of 16 short tiles: measured 14.4 us, 4 splits 16.3), and so does
-    # twice that batch (14.4 us, 4 splits 22.0); so do half as many slices of twice the length, where work-groups of 32
-    # rows whose waves share out the key tiles serve the unsplit launch (with the 128-row instances it would split 4
-    # ways), while few rows in front of long keys still split; the prefill benchmark shapes stay unsplit
+    # twice that batch (14.4 us, 4 splits 22.0); so do half as many slices of twice the length at d = 63, where work-groups
+    # of 32 rows whose waves share out the key tiles serve the unsplit launch (with the 128-row instances it would split 4
+    # ways); at d = 100 those work-groups have one LDS stage per wave and wait for much of every tile request, and four
+    # splits win; few rows in front of long keys split as before; the prefill benchmark shapes stay unsplit
     assert fa.resolve_splits(1, 8, 1021, 1021, 31, 0) == 1
     assert fa.resolve_splits(2, 8, 1021, 1021, 31, 0) == 1
     assert fa.resolve_splits(1, 4, 2048, 2048, 63, 0) == 1
-    assert fa.resolve_splits(1, 4, 2048, 2048, 100, 0) == 1
-    assert fa.resolve_splits(1, 4, 2048, 2048, 100, 0, kernel_hint=fa.KERNEL_4WAVE) == 4
+    assert fa.resolve_splits(1, 4, 2048, 2048, 63, 0, kernel_hint=fa.KERNEL_4WAVE) == 4
+    assert fa.resolve_splits(1, 4, 2048, 2048, 100, 0) == 4
     assert fa.resolve_splits(1, 8, 200, 8000, 100, 0) == 16
     assert fa.resolve_splits(4, 16, 2048, 2048, 128, 0) == 1
     assert fa.resolve_splits(4, 16, 2048, 2048, 128, 0, causal=True) == 1

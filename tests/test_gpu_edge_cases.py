@@ -370,7 +370,7 @@ def test_split_index_rotation(fa, oracle, H, S):
     (1, 8, 512, 32768, 128, False, 16),   # long keys, small batch: two work-groups per CU
     (1, 32, 128, 16384, 128, True, 8),    # causal with Nq < Nk: every split holds visible keys
     (1, 8, 200, 8000, 100, False, 16),    # rows at any alignment
-    (1, 2, 8192, 8192, 64, True, None),   # causal, one work-group per CU at most: split for the heaviest row block
+    (1, 1, 16384, 16384, 64, True, None), # causal, one work-group per CU at most: split for the heaviest row block
     (1, 40, 128, 8192, 128, False, 6),
 ])
 def test_automatic_split_count_shapes(fa, oracle, B, H, Nq, Nk, d, causal, want):
