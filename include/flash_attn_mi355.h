@@ -93,7 +93,8 @@ typedef struct flash_params {
      * feature and head dim, which is about 20 % slower.  No counterpart in the reference. */
     float *scores_out;
     /* Which tiled kernel serves the call, for A/B measurements and tests: 0 = the library chooses (by shape),
-     * 1 = the 4-wave kernel (128 query rows per work-group), 2 = the 8-wave ping-pong kernel (256 rows; needs
+     * 1 = the 4-wave kernel with 128 query rows per work-group (left to itself the library gives small unsplit
+     * problems work-groups of 32 rows whose waves share out the key tiles), 2 = the 8-wave ping-pong kernel (256 rows; needs
      * 96 < d <= 128, a positive scale and more than 128 query rows, and is ignored otherwise).  Any other value: FLASH_EINVAL.
      * The reference selects its kernel by template flags alone (src/main.cu:141-178) and has no such switch. */
     int kernel_hint;
