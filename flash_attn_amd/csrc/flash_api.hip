@@ -188,8 +188,8 @@ long long tiled_groups(const flash_params* p, const fa::FwdArgs& a)
 //    (B1 H2 N16384 d64: 194 us unsplit, 124 us in 5 splits; B1 H16 N2048 d128 stays unsplit: 39 us against 44).
 // The estimate for s splits: k (a + b t) / rho + [s > 1] (c0 + s * partials), t = tiles of a work-group (the heaviest one
 // plus k - 1 average ones), b = microseconds per 64-key tile of a work-group alone on its CU, rho the gain of k side by
-// side.  Over 21 swept shapes the count it picks is within 5 % of the best measured one on 19 (the others: 5.4 % and
-// 15 %); the reference's rule with 256 CUs: 12 of 21, the worst 6.8 times slower than the best count.
+// side.  Over 21 swept shapes the count it picks is within 5 % of the best measured one on 19 (the others: 6 % and
+// 9 %); the reference's rule with 256 CUs: 9 of 21, the worst 3.1 times slower than the best count.
 int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode);
 
 // The estimate walks the row blocks once per candidate count (up to 0.26 ms on a causal sequence of 65536 rows), and
