@@ -219,6 +219,45 @@ def test_row_blocks_without_visible_keys(fa, oracle, d):
     check_o_lse(o1, l1, O1, L1, f"d={d} two rows, one key")
 
 
+def test_concurrent_callers_on_their_own_streams(fa):
+    """Four host threads, each with a stream of its own, call the library at the same time (ctypes releases the
+    interpreter lock for the duration of a call) on different shapes -- both tiled kernels, 32-row work-groups, decode,
+    split + combine with the automatic count, whose answers each thread remembers for itself.  Results must be bit-identical
+    to the same calls made one after the other."""
+    import threading
+    import torch
+    shapes = [(1, 8, 1021, 1021, 31, dict()), (2, 16, 512, 512, 128, dict(causal=True)), (4, 16, 1, 4096, 64, dict()),
+              (1, 4, 300, 9000, 96, dict(causal=True)), (2, 8, 700, 700, 128, dict(kernel_hint=fa.KERNEL_8WAVE)),
+              (1, 2, 2048, 2048, 64, dict(causal=True)), (1, 6, 100, 3000, 40, dict(window=(500, 20))),
+              (8, 8, 256, 256, 80, dict())]
+    inputs = [tuple(randn_f16_gpu(sz, 900 + 3 * n + j) for j, sz in enumerate(((B, H, Nq, d), (B, H, Nk, d), (B, H, Nk, d))))
+              for n, (B, H, Nq, Nk, d, kw) in enumerate(shapes)]
+    want = [fa.flash_forward_splitkv(*qkv, num_splits=0, **sh[5]) for qkv, sh in zip(inputs, shapes)]
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(t):
+        try:
+            st = torch.cuda.Stream()
+            with torch.cuda.stream(st):
+                for rep in range(6):
+                    for n in range(len(shapes)):
+                        m = (n + 2 * t + rep) % len(shapes)
+                        o, lse = fa.flash_forward_splitkv(*inputs[m], num_splits=0, stream=st, **shapes[m][5])
+                        st.synchronize()
+                        if not (torch.equal(o, want[m][0]) and torch.equal(lse, want[m][1])):
+                            errors.append((t, rep, m))
+        except Exception as e:  # noqa: BLE001 -- reported by the assertion below
+            errors.append((t, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_many_head_slices_in_chunks(fa, oracle, causal):
     """With far more work-groups than the GPU holds at once the kernels deal the head slices out in chunks (here 256
