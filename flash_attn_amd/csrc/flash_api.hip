@@ -167,7 +167,7 @@ int launch_tiled(const flash_params* p, const fa::FwdArgs& a, hipStream_t st)
 // work-groups of the tiled launch for the (final) arguments a
 long long tiled_groups(const flash_params* p, const fa::FwdArgs& a)
 {
-    const bool pp = a.d > 96 && fa::fwd_uses_pingpong(a.d, !needs_every_instance(p), a.Nq, a.causal, a.wl, a.wr,
+    const bool pp = a.d > 96 && fa::fwd_uses_pingpong(a.d, !needs_every_instance(p), a.Nq, a.Nk, a.causal, a.wl, a.wr,
                                                       (long long)a.B * a.H * a.num_splits, a.kernel_hint);
     const int rows = pp ? 256 : kRowsPerGroup;
     return (long long)((a.Nq + rows - 1) / rows) * a.B * a.H * a.num_splits;
@@ -223,7 +223,7 @@ int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode)
 {
     const int wl = window_left_of(p), wr = window_right_of(p);
     const bool every = needs_every_instance(p);
-    const bool pp = fa::fwd_uses_pingpong(p->d, !every, p->Nq, p->is_causal, wl, wr, (long long)p->B * p->H, p->kernel_hint);
+    const bool pp = fa::fwd_uses_pingpong(p->d, !every, p->Nq, p->Nk, p->is_causal, wl, wr, (long long)p->B * p->H, p->kernel_hint);
     const int rows = pp ? 256 : kRowsPerGroup;
     const int Tr = (p->Nq + rows - 1) / rows;
     const long long slices = (long long)p->B * p->H;
@@ -299,12 +299,12 @@ int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode)
         if (s == 1 && narrow) {
             // 32-row work-groups with a visible key, and the time per tile of a wave on its own, measured: x 1.15 with
             // two LDS stages per wave (d <= 64); with one, where the next tile's requests are only partly hidden, x 1.3 at
-            // d = 96, x 1.6 at d = 128 and x 2.1 for rows shorter than the bucket; work-groups that follow another on
+            // d = 96 and x 1.6 at d = 128 (rows shorter than those buckets do not take these instances); work-groups that follow another on
             // their CU find their tiles in L2 and take half of that
             const long long gn = (groups * ((p->Nq + 31) / 32) + Tr - 1) / Tr;
             const long long kn = (gn + kNumCU - 1) / kNumCU;
             const float rhon = kn >= 2 && p->d <= 32 ? rho2 : 1.0f;
-            const float bn = (p->d <= 64 ? 1.15f : !dma ? 2.1f : bucket == 3 ? 1.3f : 1.6f) * b;
+            const float bn = (p->d <= 64 ? 1.15f : bucket == 3 ? 1.3f : 1.6f) * b;
             t = (3.0f + (float)kn * (a - 1.0f) + bn * ((float)((tmax + 3) / 4) + 0.5f * (float)(kn - 1) * (float)tiles / (float)groups / 4.0f)) / rhon;
         }
         if (s > 1) t += c0 + (float)s * (c1 + partials);

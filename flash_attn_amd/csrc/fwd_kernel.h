@@ -1025,7 +1025,7 @@ int launch_fwd_d96(const FwdArgs& a, int variant, int nb, hipStream_t st);
 int launch_fwd_d128(const FwdArgs& a, int variant, int nb, hipStream_t st);
 // whether launch_fwd_d128 takes the 8-wave kernel (256 query rows per work-group instead of 128)
 // (slices = B * H * num_splits; hint = flash_params::kernel_hint)
-bool fwd_uses_pingpong(int d, bool direct, int Nq, int causal, int wl, int wr, long long slices, int hint);
+bool fwd_uses_pingpong(int d, bool direct, int Nq, int Nk, int causal, int wl, int wr, long long slices, int hint);
 
 // Head slices per chunk of the work-group order: the smallest divisor of the slice count (a multiple of 8, which keeps a
 // slice on one XCD) whose chunk still holds twice the work-groups that run at once -- enough for "heaviest row blocks
@@ -1089,6 +1089,9 @@ inline bool fwd_uses_narrow(const FwdArgs& a, int variant, bool every)
     if (every || a.num_splits != 1 || a.stamps != nullptr || a.kernel_hint != 0) return false;
     const long long groups = (long long)a.B * a.H * ((a.Nq + 127) / 128);
     if (2 * groups > kNumCus) return false;
+    // (above d = 64 a wave has one LDS stage and waits for most of every tile request: rows shorter than the bucket,
+    // whose requests take longer, measured slower than the 128-row instances there)
+    if (a.d > 64 && a.d % 32 != 0) return false;
     const int keys = 4 * groups <= kNumCus ? 512 : 1024;  // visible keys per row that make the chain worth cutting
     return a.Nk >= keys && (a.wl < 0 || a.wl >= keys - 64);
 }
@@ -1129,9 +1132,11 @@ inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
             if (feat == kVarAlibi) return (int)launch_fwd_narrow_instance<D, kVarAlibi>(a, st);
             if (feat == kVarDropout) return (int)launch_fwd_narrow_instance<D, kVarDropout>(a, st);
             if (feat != 0) return (int)launch_fwd_narrow_instance<D, kVarAlibi | kVarDropout>(a, st);
-            if (!(variant & kVarVec)) return (int)launch_fwd_narrow_instance<D, 0>(a, st);
             if (a.d == D) return (int)launch_fwd_narrow_instance<D, kVarVec | kVarFullD>(a, st);
-            return (int)launch_fwd_narrow_instance<D, kVarVec>(a, st);
+            if constexpr (D <= 64) {  // (above, only rows of the bucket's width come here)
+                if (!(variant & kVarVec)) return (int)launch_fwd_narrow_instance<D, 0>(a, st);
+                return (int)launch_fwd_narrow_instance<D, kVarVec>(a, st);
+            }
         }
     }
     if (!(variant & kVarVec)) {
