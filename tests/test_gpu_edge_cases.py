@@ -117,8 +117,12 @@ def test_8wave_kernel_on_shorter_rows(fa, oracle, d):
     (2, 2, 2, 515, 515, 56, dict(causal=True, window=(600, -1))),
     (1, 5, 5, 640, 640, 32, dict(window=(-1, 64))),
     (1, 4, 4, 1, 3000, 20, dict(dropout_p=0.0)),            # one row: the decode kernel, not these instances
-    # above d = 64 a wave has one LDS stage and requests K and V of its next tile separately
+    # above d = 64 a wave has one LDS stage and requests K and V of its next tile separately (rows of the bucket's
+    # width only: the shorter rows in this list run the 128-row instances)
     (1, 8, 8, 1024, 1024, 128, dict(causal=True)),
+    (1, 4, 2, 777, 1100, 96, dict(window=(1000, 20))),
+    (1, 2, 2, 600, 700, 128, dict(causal=True, dropout_p=0.3, seed=9, offset=2)),
+    (1, 3, 1, 70, 2100, 128, dict(alibi=True)),
     (1, 4, 2, 777, 1100, 100, dict(window=(1000, 20))),
     (2, 2, 2, 515, 515, 96, dict(alibi=True)),
     (1, 3, 3, 900, 600, 127, dict(causal=True)),
