@@ -14,8 +14,11 @@
 //    head-dim column per lane: that is what ds_read_b64_tr_b16 delivers from the row-major V tile.
 //  * O^T accumulates in registers (fp32) and is normalised once in the epilogue; the reference keeps O in shared
 //    memory and renormalises it every tile (src/flash_forward.h:284-289).
-//  * K and V tiles are double-buffered in LDS; the global loads of tile t+1 are issued before the MFMA work of
-//    tile t and written to the other buffer afterwards, one barrier per tile.
+//  * K and V tiles are double-buffered in LDS and requested straight into it (global_load_lds_dwordx4), tile t+1
+//    while tile t is computed, one barrier per tile; only the instance that serves every request (rows of fewer than
+//    eight elements among them) stages its tiles through registers.
+//  * Small unsplit problems take the narrow instances: 32 query rows per work-group, held by all four waves, each of
+//    which walks every fourth key tile with LDS stages of its own; the four results are merged through LDS.
 //  * Every mask of the family (causal, sliding window, key bound for ragged Nk) is one per-row interval
 //    [lo_i, hi_i] of allowed keys; tiles entirely inside the interval of every row of the wave skip the
 //    element test.  The KV tile range of the group is pruned like src/flash_forward.h:39-48.
