@@ -1093,8 +1093,10 @@ inline bool fwd_uses_narrow(const FwdArgs& a, int variant, bool every)
     const long long groups = (long long)a.B * a.H * ((a.Nq + 127) / 128);
     if (2 * groups > kNumCus) return false;
     // (above d = 64 a wave has one LDS stage and waits for most of every tile request: rows shorter than the bucket,
-    // whose requests take longer, measured slower than the 128-row instances there)
-    if (a.d > 64 && a.d % 32 != 0) return false;
+    // whose requests take longer, measured slower than the 128-row instances there, and so did launches of more 32-row
+    // work-groups than CUs unless causal -- B2 H2 Nq4096 Nk1024 d128 25.6 against 20.9 us, the same causal shapes 39.5
+    // against 69.0 us)
+    if (a.d > 64 && (a.d % 32 != 0 || (!a.causal && (long long)a.B * a.H * ((a.Nq + 31) / 32) > kNumCus))) return false;
     const int keys = 4 * groups <= kNumCus ? 512 : 1024;  // visible keys per row that make the chain worth cutting
     return a.Nk >= keys && (a.wl < 0 || a.wl >= keys - 64);
 }
@@ -1130,11 +1132,13 @@ inline int launch_fwd_bucket_st(const FwdArgs& a, int variant, hipStream_t st)
     constexpr int AL = kVarAlibi | kVarAlibiLeft;  // ALiBi with no visible key right of its row
     if constexpr (ST == 0) {
         if (fwd_uses_narrow(a, variant, fwd_needs_every_instance(a, variant))) {
-            // plain: by row length like the others; with ALiBi or dropout: the instances for rows at any alignment,
-            // which serve every row length from eight elements on
-            if (feat == kVarAlibi) return (int)launch_fwd_narrow_instance<D, kVarAlibi>(a, st);
-            if (feat == kVarDropout) return (int)launch_fwd_narrow_instance<D, kVarDropout>(a, st);
-            if (feat != 0) return (int)launch_fwd_narrow_instance<D, kVarAlibi | kVarDropout>(a, st);
+            // plain: by row length like the others; with ALiBi or dropout: up to d = 64 the instances for rows at any
+            // alignment, which serve every row length from eight elements on, above the ones for rows of the bucket's
+            // width (the only rows that come here)
+            constexpr int F = D <= 64 ? 0 : kVarVec | kVarFullD;
+            if (feat == kVarAlibi) return (int)launch_fwd_narrow_instance<D, F | kVarAlibi>(a, st);
+            if (feat == kVarDropout) return (int)launch_fwd_narrow_instance<D, F | kVarDropout>(a, st);
+            if (feat != 0) return (int)launch_fwd_narrow_instance<D, F | kVarAlibi | kVarDropout>(a, st);
             if (a.d == D) return (int)launch_fwd_narrow_instance<D, kVarVec | kVarFullD>(a, st);
             if constexpr (D <= 64) {  // (above, only rows of the bucket's width come here)
                 if (!(variant & kVarVec)) return (int)launch_fwd_narrow_instance<D, 0>(a, st);
