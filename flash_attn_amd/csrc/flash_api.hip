@@ -299,13 +299,16 @@ int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode)
         if (s == 1 && narrow) {
             // 32-row work-groups with a visible key, and the time per tile of a wave on its own, measured: x 1.15 with
             // two LDS stages per wave (d <= 64); with one, where the next tile's requests are only partly hidden, x 1.3 at
-            // d = 96 and x 1.6 at d = 128 (rows shorter than those buckets do not take these instances); work-groups that follow another on
-            // their CU find their tiles in L2 and take half of that
+            // d = 96 and x 1.6 at d = 128 (rows shorter than those buckets do not take these instances), x 1.7 on top for
+            // odd d (every second row off a 4-byte boundary: slower requests, which a wave on its own cannot hide); under
+            // a causal mask with about as many rows as keys the work-groups that follow another on their CU are the
+            // light ones of rows that found their tiles in L2 already, and take half of that
             const long long gn = (groups * ((p->Nq + 31) / 32) + Tr - 1) / Tr;
             const long long kn = (gn + kNumCU - 1) / kNumCU;
             const float rhon = kn >= 2 && p->d <= 32 ? rho2 : 1.0f;
-            const float bn = (p->d <= 64 ? 1.15f : bucket == 3 ? 1.3f : 1.6f) * b;
-            t = (3.0f + (float)kn * (a - 1.0f) + bn * ((float)((tmax + 3) / 4) + 0.5f * (float)(kn - 1) * (float)tiles / (float)groups / 4.0f)) / rhon;
+            const float bn = (p->d <= 64 ? 1.15f : bucket == 3 ? 1.3f : 1.6f) * ((p->d & 1) ? 1.7f : 1.0f) * b;
+            const float later = p->is_causal && 2 * p->Nq >= p->Nk ? 0.5f : 1.0f;
+            t = (3.0f + (float)kn * (a - 1.0f) + bn * ((float)((tmax + 3) / 4) + later * (float)(kn - 1) * (float)tiles / (float)groups / 4.0f)) / rhon;
         }
         if (s > 1) t += c0 + (float)s * (c1 + partials);
         if (s == 1 || t < best_t) {
