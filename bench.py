@@ -65,6 +65,8 @@ DIAG = {
     "diag_split_long_keys": dict(B=1, H=8, Nq=512, Nk=32768, d=128, causal=False, window=(-1, -1), alibi=False, p=0.0, splits=-1),
     "diag_split_causal": dict(B=1, H=32, Nq=128, Nk=16384, d=128, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=-1),
     "diag_split_ref_default": dict(B=2, H=8, Nq=1021, Nk=1021, d=31, causal=False, window=(-1, -1), alibi=False, p=0.0, splits=-1),
+    # the reference's own run (src/main.cu:39-49) with the library's split count: one launch of 32-row work-groups
+    "diag_ref_default": dict(B=1, H=8, Nq=1021, Nk=1021, d=31, causal=False, window=(-1, -1), alibi=False, p=0.0, splits=-1),
     # grouped-query prefill: the query heads of a K/V head read the same K and V
     "diag_gqa_prefill": dict(B=4, H=32, Hk=4, Nq=4096, Nk=4096, d=128, causal=True, window=(-1, -1), alibi=False, p=0.0, splits=0),
 }
@@ -86,6 +88,7 @@ DESCR = {
     "diag_split_long_keys": "split-KV fwd, automatic split count, B=1 H=8 Nq=512 Nk=32768 d=128 (diagnostic)",
     "diag_split_causal": "split-KV causal fwd, automatic split count, B=1 H=32 Nq=128 Nk=16384 d=128 (diagnostic)",
     "diag_split_ref_default": "split-KV fwd, automatic split count, B=2 H=8 Nq=Nk=1021 d=31 (diagnostic)",
+    "diag_ref_default": "split-KV fwd, automatic split count, B=1 H=8 Nq=Nk=1021 d=31: the reference's own run (diagnostic)",
     "diag_gqa_prefill": "causal fwd, 8 query heads per K/V head, B=4 H=32 H_kv=4 Nq=Nk=4096 d=128 (diagnostic)",
 }
 
