@@ -210,7 +210,8 @@ int auto_splits_tiled(const flash_params* p, int n_blocks, bool decode = false)
     static thread_local int next = 0;
     const Key key = {p->B, p->H, p->H_kv, p->Nq, p->Nk, p->d, p->is_causal, window_left_of(p), window_right_of(p), p->kernel_hint,
                      tiled_variant(p) | (p->softmax_scale > 0.0f ? 8 : 0) | (p->scores_out ? 16 : 0) | (decode ? 32 : 0) |
-                         (p->dropout_p > 0.0f && flash_dropout_threshold(p->dropout_p) == 0 ? 64 : 0)};
+                         (p->dropout_p > 0.0f && flash_dropout_threshold(p->dropout_p) == 0 ? 64 : 0) |
+                         (p->stage_stamps_out ? 128 : 0)};
     for (const Entry& e : memo)
         if (e.valid && e.key == key) return e.splits;
     const int splits = auto_splits_tiled_uncached(p, n_blocks, decode);
