@@ -342,7 +342,7 @@ __device__ __forceinline__ v4u philox4x32_10_c2(uint32_t c0, uint32_t c1, uint32
                                                 uint32_t k1)
 {
     uint32_t hi0, lo0, hi1, lo1;
-    // round 1
+    // first Philox round
     mul_wide_u32(0xD2511F53u, c0, hi0, lo0);
     uint32_t n0 = c1 ^ (c2_hi ^ k0);
     const uint32_t u1 = c2_lo;  // uniform
@@ -350,7 +350,7 @@ __device__ __forceinline__ v4u philox4x32_10_c2(uint32_t c0, uint32_t c1, uint32
     uint32_t n3 = lo0;
     k0 += 0x9E3779B9u;
     k1 += 0xBB67AE85u;
-    // round 2: its second word is still uniform
+    // second Philox round: its second word is still uniform
     mul_wide_u32(0xD2511F53u, n0, hi0, lo0);
     mul_wide_u32(0xCD9E8D57u, n2, hi1, lo1);
     c0 = hi1 ^ (u1 ^ k0);
