@@ -230,15 +230,16 @@ int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode)
     const long long slices = (long long)p->B * p->H;
     if (slices * Tr >= 4LL * kNumCU) return 1;  // (the reference's early exit: four rounds of work-groups as they are)
     const int bucket = (p->d + 31) / 32;  // head-dim bucket of the kernel instance: 1 ... 4
-    // microseconds per tile of a lone work-group, by bucket; x 1.05 for rows that are not the bucket's width (chunk
-    // positions past the row are fetched and multiplied all the same; rows at any alignment, d % 8 != 0, measured
-    // 1.0-1.2 x the bucket-wide instance), x 1.5 for the instance that serves every request (tiles staged through
-    // registers)
+    // microseconds per tile of a lone work-group, by bucket; x 1.5 for the instance that serves every request (tiles
+    // staged through registers)
     static const float kTile[5] = {0.0f, 0.5f, 0.72f, 0.88f, 1.0f};
     const bool dma = !every && p->d == 32 * bucket;
     // (decode launches, whose tiles no other work-group has asked for before: twice that, and 0.04 us per split for
     // the combine of their few rows; fitted to 55 random decode shapes of the tiled routes)
-    const float b = (pp ? 1.97f : kTile[bucket] * (dma ? 1.0f : every ? 1.5f : 1.05f)) * (decode ? 2.0f : 1.0f);
+    // (rows shorter than the bucket fetch and multiply past their end, but fewer bytes arrive: measured d = 72 at 0.86 of
+    // d = 96 per tile, d = 100 at 0.9 of 128)
+    const float shorter = (0.55f + 0.45f * (float)p->d / (float)(32 * bucket)) * ((p->d & 7) ? 1.05f : 1.0f);
+    const float b = (pp ? 1.97f : kTile[bucket] * (dma ? 1.0f : every ? 1.5f : shorter)) * (decode ? 2.0f : 1.0f);
     const float rho2 = pp ? 1.0f : every ? 1.4f : 1.32f;
     const float rho3 = (!pp && !every && p->d <= 64) ? rho2 * 1.12f : rho2;  // three places per CU up to d = 64
     // a: prologue + epilogue of a work-group; c0 + c1 s: the combine launch and what every further split adds to it and to
