@@ -186,9 +186,10 @@ long long tiled_groups(const flash_params* p, const fa::FwdArgs& a)
 //  * under a causal mask the launch takes as long as its heaviest work-group, the last row block's longest split, alone
 //    on its CU for most of its life: with few head slices splitting shortens exactly that
 //    (B1 H2 N16384 d64: 194 us unsplit, 124 us in 5 splits; B1 H16 N2048 d128 stays unsplit: 39 us against 44).
-// The estimate for s splits: k (a + b t) / rho + [s > 1] (c0 + s * partials), t = tiles of a work-group (the heaviest one
-// plus k - 1 average ones), b = microseconds per 64-key tile of a work-group alone on its CU, rho the gain of k side by
-// side.  Over 21 swept shapes the count it picks is within 5 % of the best measured one on 19 (the others: 6 % and
+// The estimate for s splits: k a / rho + b t + [s > 1] (c0 + s * partials), k = work-groups on the fullest CU, t = their
+// tiles (the heaviest one plus k - 1 average ones) taken in rounds of as many as the CU has places for, a round of n
+// side by side costing the sum of its tiles over the gain of n, b = microseconds per 64-key tile of a work-group alone
+// on its CU.  Over 21 swept shapes the count it picks is within 5 % of the best measured one on 19 (the others: 6 % and
 // 9 %); the reference's rule with 256 CUs: 9 of 21, the worst 3.1 times slower than the best count.
 int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode);
 
@@ -297,7 +298,18 @@ int auto_splits_tiled_uncached(const flash_params* p, int n_blocks, bool decode)
         if (groups == 0) return 1;
         const long long k = (groups + kNumCU - 1) / kNumCU;
         const float rho = k == 1 ? 1.0f : k == 2 ? rho2 : rho3;
-        float t = ((float)k * a + b * ((float)tmax + (float)(k - 1) * (float)tiles / (float)groups)) / rho;
+        // The k work-groups of the fullest CU run `places` at a time: whole rounds side by side, and what is left over
+        // in a last round with less company (three work-groups on two places take a round of two and a round of one).
+        const int places = pp ? 1 : (!every && p->d <= 64) ? 3 : 2;
+        const float avg = (float)tiles / (float)groups;
+        const float gain[4] = {1.0f, 1.0f, rho2, rho3};
+        float chain = 0.0f;  // tiles of the fullest CU, in units of a lone work-group's tile
+        for (long long left = k; left > 0;) {
+            const int n = left < places ? (int)left : places;
+            chain += ((left == k ? (float)tmax + (float)(n - 1) * avg : (float)n * avg)) / gain[n];
+            left -= n;
+        }
+        float t = (float)k * a / rho + b * chain;
         if (s == 1 && narrow) {
             // 32-row work-groups with a visible key, and the time per tile of a wave on its own, measured: x 1.15 with
             // two LDS stages per wave (d <= 64); with one, where the next tile's requests are only partly hidden, x 1.3 at
